@@ -11,6 +11,7 @@ from .registry import (
     register_architecture,
 )
 from .spec import LayerRun, LayerSpec, ModelSpec, PartSpec
+from .vepitar import VepitarConfig
 from .zabunex import ZabunexConfig
 
 __all__ = [
@@ -26,6 +27,7 @@ __all__ = [
     "ModelSpec",
     "PartSpec",
     "ServerConfig",
+    "VepitarConfig",
     "ZabunexConfig",
     "get_architecture",
     "parse_config",

@@ -386,7 +386,7 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
                         j0 >= lo_last[rt];
       // (RULED: sv holds scaled scores, in units of log2, with the bias added)
       const bool far = RULED && p_first[rt] - (j0 + KB - 1) >= rule.bias_len - 1;  // (the same for the wave)
-      auto ruled = [&](float raw, int j) {
+      auto biased = [&](float raw, int j) {
         if constexpr (RULED) {
           if (rule.bias == nullptr) return raw * scale_log2e;
           if (far) return __builtin_fmaf(raw, scale_log2e, far_bias[rt]);
@@ -396,6 +396,15 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
         } else {
           return raw;
         }
+      };
+      // (weights that are sigmoids: the score becomes log2 sigmoid, so that 2^(score - m) is
+      // the weight relative to 2^m as for a softmax)
+      auto ruled = [&](float raw, int j) {
+        float x = biased(raw, j);
+        if constexpr (RULED) {
+          if (rule.sink == HAL_WEIGHTS_SIGMOID) x = fminf(x, 0.f) - __log2f(1.0f + fast_exp2(-fabsf(x)));
+        }
+        return x;
       };
       if (full) {  // every key of the step is visible to every row of the tile
 #pragma unroll
@@ -878,9 +887,12 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
     if (!row_ok[rt]) continue;
     if (partial < 0 || merged_here) {
       if constexpr (RULED) {
-        if (rule.sink && m[rt] != -INFINITY) lt += exp2f(-m[rt]);  // (sums are relative to 2^m)
+        if (rule.sink == HAL_WEIGHTS_SINK && m[rt] != -INFINITY) lt += exp2f(-m[rt]);  // (sums are relative to 2^m)
       }
-      const float inv = lt > 0.f ? 1.0f / lt : 0.f;
+      float inv = lt > 0.f ? 1.0f / lt : 0.f;
+      if constexpr (RULED) {
+        if (rule.sink == HAL_WEIGHTS_SIGMOID) inv = m[rt] != -INFINITY ? exp2f(m[rt]) : 0.f;  // (not normalised)
+      }
       bf16_t* op = out + (size_t)(q_start + qi[rt]) * out_row_stride + (size_t)head[rt] * D;
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) {
@@ -984,8 +996,9 @@ attention_merge_kernel(bf16_t* __restrict__ out, int out_row_stride,
   float l_sum = 0.f;
 #pragma unroll
   for (int w = 0; w < MW; ++w) l_sum += red_l[w];
-  if (sink && m_all != -INFINITY) l_sum += exp2f(-m_all);
-  const float inv = l_sum > 0.f ? 1.0f / l_sum : 0.f;
+  if (sink == HAL_WEIGHTS_SINK && m_all != -INFINITY) l_sum += exp2f(-m_all);
+  float inv = l_sum > 0.f ? 1.0f / l_sum : 0.f;
+  if (sink == HAL_WEIGHTS_SIGMOID) inv = m_all != -INFINITY ? exp2f(m_all) : 0.f;
   const int qi = rho / G, head = g * G + rho % G;
   bf16_t* op = out + (size_t)(q_start + qi) * out_row_stride + (size_t)head * D;
 #pragma unroll
@@ -1041,8 +1054,9 @@ attention_merge_few_kernel(bf16_t* __restrict__ out, int out_row_stride,
       acc[c][1] += w * v.y;
     }
   }
-  if (sink && m_all != -INFINITY) l_all += exp2f(-m_all);
-  const float inv = l_all > 0.f ? 1.0f / l_all : 0.f;
+  if (sink == HAL_WEIGHTS_SINK && m_all != -INFINITY) l_all += exp2f(-m_all);
+  float inv = l_all > 0.f ? 1.0f / l_all : 0.f;
+  if (sink == HAL_WEIGHTS_SIGMOID) inv = m_all != -INFINITY ? exp2f(m_all) : 0.f;
   const int qi = rho / G, head = g * G + rho % G;
   bf16_t* op = out + (size_t)(q_start + qi) * out_row_stride + (size_t)head * D;
 #pragma unroll
@@ -1115,7 +1129,8 @@ extern "C" int hal_attention_mfma_ruled(const void* q, int q_row_stride, void* o
                                         int merge_parts, hipStream_t stream) {
   HAL_REQUIRE(chunk >= 0 && (bias_log2 == nullptr || bias_len > 0),
               "hal_attention_mfma: chunk %d, bias table of %d distances", chunk, bias_len);
-  const hal_score_rule rule = {window, chunk, bias_len, sink ? 1 : 0, bias_log2};
+  HAL_REQUIRE(sink >= HAL_WEIGHTS_SOFTMAX && sink <= HAL_WEIGHTS_SIGMOID, "hal_attention_mfma: weights of kind %d", sink);
+  const hal_score_rule rule = {window, chunk, bias_len, sink, bias_log2};
   const bool ruled = bias_log2 != nullptr || sink;
   HAL_REQUIRE(head_dim == D, "hal_attention_mfma: built for head size %d, called with %d", D,
               head_dim);

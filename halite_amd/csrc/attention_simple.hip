@@ -356,6 +356,7 @@ attention_plain_kernel(const T* __restrict__ q, int q_row_stride, T* __restrict_
             }
             if (valid) s = dot * scale;
             if (valid && rule.bias) s += hal_rule_bias(rule, h_first + r % heads_here, p - j);
+            if (valid && rule.sink == HAL_WEIGHTS_SIGMOID) s = hal_log_sigmoid(s);
           }
           const float m_new = fmaxf(m[rr], plain_wave_max(s));
           // (a NaN score makes every sum NaN, as it must; m_new is -inf only if no key is valid)
@@ -637,6 +638,7 @@ attention_rows_kernel(const T* __restrict__ q, int q_row_stride, T* __restrict__
         const int j = j0 + 8 * (v / 4) + 4 * half + v % 4;
         valid[v] = j >= lo && j <= p;
         st[v] = valid[v] ? st[v] * scale + (rule.bias ? hal_rule_bias(rule, head, p - j) : 0.f) : -INFINITY;
+        if (valid[v] && rule.sink == HAL_WEIGHTS_SIGMOID) st[v] = hal_log_sigmoid(st[v]);
         mx = fmaxf(mx, st[v]);
       }
       {
@@ -767,7 +769,8 @@ extern "C" int hal_attention_simple_ruled(const void* q, int q_row_stride, void*
                                           hipStream_t stream) {
   HAL_REQUIRE(chunk >= 0 && (bias == nullptr || bias_len > 0),
               "hal_attention_simple: chunk %d, bias table of %d distances", chunk, bias_len);
-  const hal_score_rule rule = {window, chunk, bias_len, sink ? 1 : 0, bias};
+  HAL_REQUIRE(sink >= HAL_WEIGHTS_SOFTMAX && sink <= HAL_WEIGHTS_SIGMOID, "hal_attention_simple: weights of kind %d", sink);
+  const hal_score_rule rule = {window, chunk, bias_len, sink, bias};
   HAL_REQUIRE(n_tokens >= 0 && H > 0 && K > 0 && D > 0 && page_size > 0 && n_pages > 0,
               "hal_attention_simple: bad sizes T=%d H=%d K=%d D=%d page=%d pages=%d", n_tokens, H,
               K, D, page_size, n_pages);

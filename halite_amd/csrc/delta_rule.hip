@@ -1,0 +1,220 @@
+// The generalized delta rule: per head a float32 state S [key channel][value channel] that
+// every token decays per key channel, erases along its unit key and writes to,
+//
+//   S_t = diag(w_t) S_(t-1) - (a_t * u_t) (u_t^T S_(t-1)) + k_t v_t^T,   o_t = S_t^T r_t,
+//   w = exp(-e^(-1/2) sigmoid(w0 + W2 tanh(x1))),  a = sigmoid(a_raw + a_bias),
+//   u = k / sqrt(sum(k^2) + 1e-6)   (per head),
+//
+// where both middle terms read the old state.  The state lives in float32 rows, one per
+// request slot, and a step's tokens come as a flat batch of segments, as for the other
+// recurrences.  Three kernels: what a token contributes (decay, erase vector, unit key; all
+// tokens side by side), the walk over the tokens of every segment, and the norm and gate of
+// the walk's result.  Everything here is float32 whatever the activations' type is.
+#include "hal_common.h"
+#include "hal_api.h"
+
+#define DELTA_MAX_LORA 1024
+#define DELTA_VECTORS 5  // per token and head: decay, a * u, u, k, r
+
+__device__ __forceinline__ float delta_sigmoid(float x) { return 1.0f / (1.0f + expf(-x)); }
+
+// ---- a workgroup a (token, head); thread c a key channel.  pre [T][H][5][DP], zero beyond D.
+__global__ void delta_prep_kernel(const float* __restrict__ r, int ldr, const float* __restrict__ k, int ldk,
+                                  const float* __restrict__ a_raw, int lda, const float* __restrict__ x1, int ldx1,
+                                  const void* __restrict__ w2, const void* __restrict__ w0,
+                                  const void* __restrict__ a_bias, int w_dtype, int lora, float decay_rate,
+                                  float unit_eps, float* __restrict__ pre, int H, int D, int DP) {
+  __shared__ float scratch[16];
+  __shared__ float tl[DELTA_MAX_LORA];
+  const size_t t = blockIdx.x;
+  const int h = blockIdx.y, c = threadIdx.x;
+  for (int j = threadIdx.x; j < lora; j += blockDim.x) tl[j] = tanhf(x1[t * ldx1 + j]);
+  const bool live = c < D;
+  const size_t ch = (size_t)h * D + c;
+  const float kc = live ? k[t * ldk + ch] : 0.f;
+  const float kk = block_sum(kc * kc, scratch);  // (its barrier also covers tl)
+  if (c >= DP) return;
+  float* dst = pre + ((t * H + h) * DELTA_VECTORS) * DP + c;
+  float decay = 0.f, au = 0.f, u = 0.f, rc = 0.f;
+  if (live) {
+    float z = load_as_f32(w0, w_dtype, ch);
+    for (int j = 0; j < lora; ++j) z = fmaf(load_as_f32(w2, w_dtype, ch * lora + j), tl[j], z);
+    decay = expf(-decay_rate * delta_sigmoid(z));
+    u = kc / sqrtf(kk + unit_eps);
+    au = delta_sigmoid(a_raw[t * lda + ch] + load_as_f32(a_bias, w_dtype, ch)) * u;
+    rc = r[t * ldr + ch];
+  }
+  dst[0] = decay;
+  dst[DP] = au;
+  dst[2 * DP] = u;
+  dst[3 * DP] = kc;
+  dst[4 * DP] = rc;
+}
+
+// ---- the walk: a wave takes 16 value channels of one head of one segment; the key channels
+// are split over the wave's four quarters, so a lane holds NREG numbers of its channel's
+// column of the state, and the two sums over the key channels (u^T S and S^T r) cross the
+// quarters with two exchanges each.  A token's five vectors (shared by the lanes) go through
+// LDS, the next token's on their way meanwhile.
+template <int NREG>
+__global__ void __launch_bounds__(HAL_WAVE)
+delta_scan_kernel(const float* __restrict__ pre, const float* __restrict__ v, int ldv, float* __restrict__ state,
+                  const int* __restrict__ seg_q_start, const int* __restrict__ seg_q_len,
+                  const int* __restrict__ token_slot, float* __restrict__ o, int H, int D) {
+  constexpr int DP = NREG * 4, TOTAL = DELTA_VECTORS * DP, PER = (TOTAL + HAL_WAVE - 1) / HAL_WAVE;
+  __shared__ __align__(16) float vec[2][TOTAL];
+  const int s = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int col = blockIdx.z * 16 + lane % 16, row0 = (lane / 16) * NREG;
+  const int t0 = seg_q_start[s], n = seg_q_len[s];
+  if (n <= 0) return;
+  const bool live = col < D;
+  float* st = state + ((size_t)token_slot[t0] * H + h) * D * D + (live ? col : 0);
+  float S[NREG];
+#pragma unroll
+  for (int i = 0; i < NREG; ++i) S[i] = (live && row0 + i < D) ? st[(size_t)(row0 + i) * D] : 0.f;
+
+  float next[PER];
+  auto ask = [&](int t) {
+    const float* src = pre + ((size_t)t * H + h) * TOTAL;
+#pragma unroll
+    for (int u = 0; u < PER; ++u) {
+      const int i = lane + u * HAL_WAVE;
+      next[u] = i < TOTAL ? src[i] : 0.f;
+    }
+  };
+  auto put = [&](int buf) {
+#pragma unroll
+    for (int u = 0; u < PER; ++u) {
+      const int i = lane + u * HAL_WAVE;
+      if (i < TOTAL) vec[buf][i] = next[u];
+    }
+  };
+  ask(t0);
+  float v_next = live ? v[(size_t)t0 * ldv + (size_t)h * D + col] : 0.f;
+  for (int i = 0; i < n; ++i) {
+    const int t = t0 + i, buf = i & 1;
+    put(buf);
+    const float vv = v_next;
+    if (i + 1 < n) {
+      ask(t + 1);
+      v_next = live ? v[(size_t)(t + 1) * ldv + (size_t)h * D + col] : 0.f;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const float* wv = vec[buf] + row0;
+    float d0 = 0.f, d1 = 0.f;
+#pragma unroll
+    for (int j = 0; j < NREG; j += 4) {
+      const float4 u4 = *(const float4*)(wv + 2 * DP + j);
+      d0 = fmaf(S[j], u4.x, d0);
+      d1 = fmaf(S[j + 1], u4.y, d1);
+      d0 = fmaf(S[j + 2], u4.z, d0);
+      d1 = fmaf(S[j + 3], u4.w, d1);
+    }
+    float dot = d0 + d1;  // u^T S_(t-1) of this column, a quarter of it
+    dot += __shfl_xor(dot, 16, HAL_WAVE);
+    dot += __shfl_xor(dot, 32, HAL_WAVE);
+    float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+    for (int j = 0; j < NREG; j += 4) {
+      const float4 w4 = *(const float4*)(wv + j);
+      const float4 e4 = *(const float4*)(wv + DP + j);
+      const float4 k4 = *(const float4*)(wv + 3 * DP + j);
+      const float4 r4 = *(const float4*)(wv + 4 * DP + j);
+      S[j] = fmaf(w4.x, S[j], fmaf(-e4.x, dot, k4.x * vv));
+      a0 = fmaf(S[j], r4.x, a0);
+      S[j + 1] = fmaf(w4.y, S[j + 1], fmaf(-e4.y, dot, k4.y * vv));
+      a1 = fmaf(S[j + 1], r4.y, a1);
+      S[j + 2] = fmaf(w4.z, S[j + 2], fmaf(-e4.z, dot, k4.z * vv));
+      a0 = fmaf(S[j + 2], r4.z, a0);
+      S[j + 3] = fmaf(w4.w, S[j + 3], fmaf(-e4.w, dot, k4.w * vv));
+      a1 = fmaf(S[j + 3], r4.w, a1);
+    }
+    float acc = a0 + a1;
+    acc += __shfl_xor(acc, 16, HAL_WAVE);
+    acc += __shfl_xor(acc, 32, HAL_WAVE);
+    if (live && lane < 16) o[(size_t)t * H * D + (size_t)h * D + col] = acc;
+  }
+  if (live) {
+#pragma unroll
+    for (int i = 0; i < NREG; ++i)
+      if (row0 + i < D) st[(size_t)(row0 + i) * D] = S[i];
+  }
+}
+
+// r, k, v, a_raw: float32 [T, H * D] (row-strided views allowed), x1 float32 [T, lora];
+// w2 [H * D, lora], w0 and a_bias [H * D] of one element type; state float32
+// [slots][H][D][D], read and left as the step's last state; pre: room for T * H * 5 * DP
+// floats with DP = D rounded up to 16, 32, 64, 128 or 256; o float32 [T, H * D].
+extern "C" int hal_delta_rule(const float* r, int ldr, const float* k, int ldk, const float* v, int ldv,
+                              const float* a_raw, int lda, const float* x1, int ldx1, const void* w2,
+                              const void* w0, const void* a_bias, int w_dtype, int lora, float decay_rate,
+                              float unit_eps, float* pre, float* state, const int* seg_q_start,
+                              const int* seg_q_len, const int* token_slot, float* o, int n_tokens, int n_segs,
+                              int H, int D, hipStream_t stream) {
+  HAL_REQUIRE(n_tokens >= 0 && n_segs >= 0 && H > 0 && D > 0 && lora > 0,
+              "hal_delta_rule: bad sizes T=%d segments=%d heads=%d dim=%d lora=%d", n_tokens, n_segs, H, D, lora);
+  HAL_REQUIRE(D <= 256, "hal_delta_rule: a head of %d channels exceeds 256", D);
+  HAL_REQUIRE(lora <= DELTA_MAX_LORA, "hal_delta_rule: a decay projection of rank %d exceeds %d", lora, DELTA_MAX_LORA);
+  HAL_REQUIRE(H <= 65535, "hal_delta_rule: %d heads exceed the grid limit", H);
+  HAL_REQUIRE(ldr >= H * D && ldk >= H * D && ldv >= H * D && lda >= H * D && ldx1 >= lora,
+              "hal_delta_rule: rows too short");
+  HAL_REQUIRE(w_dtype == HAL_F32 || w_dtype == HAL_BF16, "hal_delta_rule: dtype %d", w_dtype);
+  if (n_tokens == 0 || n_segs == 0) return 0;
+  const int DP = D <= 16 ? 16 : D <= 32 ? 32 : D <= 64 ? 64 : D <= 128 ? 128 : 256;
+  hipLaunchKernelGGL(delta_prep_kernel, dim3(n_tokens, H), dim3(DP < 64 ? 64 : DP), 0, stream, r, ldr, k, ldk, a_raw,
+                     lda, x1, ldx1, w2, w0, a_bias, w_dtype, lora, decay_rate, unit_eps, pre, H, D, DP);
+  const dim3 grid(n_segs, H, (D + 15) / 16);
+#define DELTA_SCAN(N_)                                                                                       \
+  hipLaunchKernelGGL(delta_scan_kernel<N_>, grid, dim3(HAL_WAVE), 0, stream, pre, v, ldv, state, seg_q_start, \
+                     seg_q_len, token_slot, o, H, D)
+  if (DP == 16) DELTA_SCAN(4);
+  else if (DP == 32) DELTA_SCAN(8);
+  else if (DP == 64) DELTA_SCAN(16);
+  else if (DP == 128) DELTA_SCAN(32);
+  else DELTA_SCAN(64);
+#undef DELTA_SCAN
+  HAL_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---- out = y / rms(y over each head) * w * sigmoid(z): a wave a (token, head) -------------
+template <typename T>
+__global__ void head_norm_gate_kernel(const float* __restrict__ y, const float* __restrict__ z, int ldz,
+                                      const void* __restrict__ w, int w_dtype, float eps, T* __restrict__ out,
+                                      int n_tokens, int H, int D) {
+  const int lane = threadIdx.x % HAL_WAVE;
+  const size_t unit = (size_t)blockIdx.x * (blockDim.x / HAL_WAVE) + threadIdx.x / HAL_WAVE;
+  if (unit >= (size_t)n_tokens * H) return;
+  const size_t t = unit / H;
+  const int h = (int)(unit % H);
+  const float* yr = y + (t * H + h) * D;
+  float ss = 0.f;
+  for (int i = lane; i < D; i += HAL_WAVE) ss += yr[i] * yr[i];
+  const float rstd = 1.0f / sqrtf(wave_sum(ss) / (float)D + eps);
+  for (int i = lane; i < D; i += HAL_WAVE) {
+    const size_t c = (size_t)h * D + i;
+    const float g = z ? delta_sigmoid(z[t * ldz + c]) : 1.0f;
+    const float wt = w ? load_as_f32(w, w_dtype, c) : 1.0f;
+    out[t * H * D + c] = from_f32<T>(yr[i] * rstd * wt * g);
+  }
+}
+
+extern "C" int hal_head_norm_gate(const float* y, const float* z, int ldz, const void* w, int w_dtype, float eps,
+                                  void* out, int dtype, int n_tokens, int H, int D, hipStream_t stream) {
+  HAL_REQUIRE(n_tokens >= 0 && H > 0 && D > 0 && (z == nullptr || ldz >= H * D),
+              "hal_head_norm_gate: bad sizes T=%d heads=%d dim=%d", n_tokens, H, D);
+  HAL_REQUIRE(dtype == HAL_F32 || dtype == HAL_BF16, "hal_head_norm_gate: dtype %d", dtype);
+  if (n_tokens == 0) return 0;
+  const long long units = (long long)n_tokens * H;
+  const dim3 grid((unsigned)((units + 3) / 4));
+  if (dtype == HAL_F32)
+    hipLaunchKernelGGL(head_norm_gate_kernel<float>, grid, dim3(256), 0, stream, y, z, ldz, w, w_dtype, eps,
+                       (float*)out, n_tokens, H, D);
+  else
+    hipLaunchKernelGGL(head_norm_gate_kernel<bf16_t>, grid, dim3(256), 0, stream, y, z, ldz, w, w_dtype, eps,
+                       (bf16_t*)out, n_tokens, H, D);
+  HAL_LAUNCH_CHECK();
+  return 0;
+}

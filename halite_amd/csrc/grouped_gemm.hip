@@ -34,6 +34,7 @@ struct GroupedArgs {
   const float* gate;   // or null
   int ldg;
   float limit, alpha;
+  int act;  // without W2: 0 the product as it is, 1 the square of its positive part
 };
 
 #define GG_ROWS 128  // rows of a workgroup's tile (what the tile offsets count in)
@@ -70,6 +71,10 @@ __device__ __forceinline__ void gg_store(const GroupedArgs& a, int g, int i, int
     const float gg = fminf(v, a.limit);
     const float uu = fminf(fmaxf(v2, -a.limit), a.limit);
     v = gg * gg_sigmoid(a.alpha * gg) * (uu + 1.0f);
+  }
+  if (!gated && a.act == 1) {
+    v = fmaxf(v, 0.f);
+    v = v * v;
   }
   const int dst = a.row_dst ? a.row_dst[i] : i;
   const size_t col = (size_t)g * a.y_group_cols + a.y_col0 + n;
@@ -355,7 +360,8 @@ extern "C" int hal_grouped_gemm(const void* X, int ldx, int x_group_cols, int x_
                                 int y_add, int M, int N, int K, int G, const int* group_offsets,
                                 const int* tile_offsets, const int* row_src, int src_div,
                                 const int* row_dst, const float* gate, int ldg, float limit,
-                                float alpha, int allow_mfma, hipStream_t stream) {
+                                float alpha, int act, int allow_mfma, hipStream_t stream) {
+  HAL_REQUIRE(act == 0 || (act == 1 && W2 == nullptr), "hal_grouped_gemm: activation %d", act);
   HAL_REQUIRE(M >= 0 && N > 0 && K > 0 && G > 0, "hal_grouped_gemm: bad sizes M=%d N=%d K=%d G=%d", M, N,
               K, G);
   HAL_REQUIRE(dtype == HAL_F32 || dtype == HAL_BF16, "hal_grouped_gemm: operand dtype %d", dtype);
@@ -374,7 +380,7 @@ extern "C" int hal_grouped_gemm(const void* X, int ldx, int x_group_cols, int x_
   a.M = M; a.N = N; a.K = K; a.G = G;
   a.group_offsets = group_offsets; a.tile_offsets = tile_offsets;
   a.row_src = row_src; a.src_div = src_div; a.row_dst = row_dst;
-  a.gate = gate; a.ldg = ldg; a.limit = limit; a.alpha = alpha;
+  a.gate = gate; a.ldg = ldg; a.limit = limit; a.alpha = alpha; a.act = act;
   const int row_tiles = (M + GG_ROWS - 1) / GG_ROWS;
   // (a list of M rows cut into G groups has at most M / tile + G tiles, each group's last one partly filled)
   dim3 grid((N + GG_TN - 1) / GG_TN * (GG_ROWS / GG_TM), group_offsets ? row_tiles + G : row_tiles,

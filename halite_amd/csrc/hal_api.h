@@ -142,13 +142,14 @@ int hal_sample_spread(const float* logits, int ld, int n_rows, int V, const floa
 // and writes row row_dst[i] of Y (i if null).  W2 != null: two products and the clamped
 // gated activation g = min(x W^T, limit), u = clamp(x W2^T, -limit, limit),
 // y = g * sigmoid(alpha * g) * (u + 1).  gate != null (float32 rows of length ldg): the
-// result is multiplied by sigmoid(gate[row, g * y_group_cols + n]).
+// result is multiplied by sigmoid(gate[row, g * y_group_cols + n]).  act (W2 null): 0 the
+// product as it is, 1 the square of its positive part.
 int hal_grouped_gemm(const void* X, int ldx, int x_group_cols, int x_col0, const void* W,
                      const void* W2, long long w_group_stride, int ldw, int dtype, void* Y, int ldy,
                      int y_group_cols, int y_col0, int y_dtype, int y_add, int M, int N, int K,
                      int G, const int* group_offsets, const int* tile_offsets, const int* row_src,
                      int src_div, const int* row_dst, const float* gate, int ldg, float limit,
-                     float alpha, int allow_mfma, hipStream_t stream);
+                     float alpha, int act, int allow_mfma, hipStream_t stream);
 
 // ---- around a latent attention and a mixture of experts (latent_moe.hip) -----------------
 // RMSNorm of rows of the float32 stream (rows[r] or r) with one or two weights, x * rstd * w
@@ -246,6 +247,44 @@ int hal_ssd_scan(const void* xbc, int ldx, int dtype, const float* dt_raw, int l
 int hal_gated_part_norm(const float* y, const float* z, int ldz, const void* w, int w_dtype,
                         float eps, void* out, int dtype, int n_tokens, int inner, int parts,
                         hipStream_t stream);
+
+// ---- the generalized delta rule (delta_rule.hip) ------------------------------------------
+// S_t = diag(w_t) S_(t-1) - (a_t * u_t)(u_t^T S_(t-1)) + k_t v_t^T, o_t = S_t^T r_t per head,
+// with w = exp(-decay_rate * sigmoid(w0 + W2 tanh(x1))), a = sigmoid(a_raw + a_bias) and
+// u = k / sqrt(sum(k^2) + unit_eps).  r, k, v, a_raw: float32 [T, H * D] (row lengths given),
+// x1 float32 [T, lora]; w2 [H * D, lora], w0 and a_bias [H * D] of element type w_dtype; state
+// float32 [slots][H][D][D], read and left as the step's last state; pre: scratch of
+// T * H * 5 * DP floats (DP: D rounded up to 16, 32, 64, 128 or 256); o float32 [T, H * D].
+int hal_delta_rule(const float* r, int ldr, const float* k, int ldk, const float* v, int ldv,
+                   const float* a_raw, int lda, const float* x1, int ldx1, const void* w2,
+                   const void* w0, const void* a_bias, int w_dtype, int lora, float decay_rate,
+                   float unit_eps, float* pre, float* state, const int* seg_q_start,
+                   const int* seg_q_len, const int* token_slot, float* o, int n_tokens, int n_segs,
+                   int H, int D, hipStream_t stream);
+// out = y / rms(y over each head of D) * w * sigmoid(z)  (w, z: null for none)
+int hal_head_norm_gate(const float* y, const float* z, int ldz, const void* w, int w_dtype, float eps,
+                       void* out, int dtype, int n_tokens, int H, int D, hipStream_t stream);
+
+// ---- several copies of the residual stream, per-head norms, per-head gates (stream_ops.hip) --
+// x float32 [S][rows][W] (copy_stride elements between copies).  With y (float32 [rows][W]):
+// x_t <- sum_s mix[s][t] x_s + m * out[t] * y for every copy t, from the old copies.  With
+// read: u = sum_s in[s] x_s (in null: ones) of the new copies, written to result as it is
+// (norm_w null, float32) or as u / sqrt(mean(u^2) + eps) * (offset + norm_w).  rows (or null;
+// only without y): the rows to take, results in that order.
+int hal_streams_step(float* x, long long copy_stride, int S, const float* y, const void* mix,
+                     const void* outw, float m, const void* inw, int c_dtype, int read,
+                     const void* norm_w, int norm_dtype, float offset, float eps, void* result,
+                     int result_dtype, const int* rows, int n_rows, int W, hipStream_t stream);
+// Every head of float32 q [T, H * dq], k [T, K * dq], v [T, K * dv] divided by its own root
+// mean square, packed as hal_qk_norm_pack packs (and appended to the pages, if given).
+int hal_head_norm_pack(const float* q, int ldq, const float* k, int ldk, const float* v, int ldv, float eps,
+                       const int* positions, void* out, int row_stride, int dtype, int n_tokens, int H,
+                       int K, int dq, int dv, int D, const int* token_seg, const int* block_table,
+                       int bt_stride, void* k_pages, void* v_pages, int page_size, int n_pages, int tiled,
+                       hipStream_t stream);
+// y[t, h * n + j] = x[t, h * x_head + j] * sigmoid(g[t, h]), j < n
+int hal_head_gate_cols(const void* x, int ldx, int x_head, const float* g, int ldg, void* y, int n, int H,
+                       int dtype, int n_tokens, hipStream_t stream);
 
 // ---- the head-size-specific library (attention_mfma.hip) ---------------------------------
 int hal_attention_mfma_head_dim();

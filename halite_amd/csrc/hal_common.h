@@ -144,7 +144,12 @@ __host__ __device__ __forceinline__ size_t kv_value_offset(bool tiled, int page_
 // chunk of that many positions (counted from position 0 of the request).  `bias` (or null):
 // float32 [heads][bias_len], added to the scaled score of a key n tokens back at
 // [head][min(n, bias_len - 1)].  `sink`: the softmax has one more term of score 0 that
-// carries no value (its denominator is 1 + the sum).
+// carries no value (its denominator is 1 + the sum); `sink` == HAL_WEIGHTS_SIGMOID: a key's
+// weight is the sigmoid of its score (scaled, bias added) and the weights are not normalised
+// over the keys.  The kernels keep their sums relative to a running maximum m either way: they
+// are handed the logarithm of the sigmoid as the score, and a finished row is multiplied by
+// exp(m) where a softmax's is divided by its sum.
+enum { HAL_WEIGHTS_SOFTMAX = 0, HAL_WEIGHTS_SINK = 1, HAL_WEIGHTS_SIGMOID = 2 };
 struct hal_score_rule {
   int window;
   int chunk;
@@ -161,9 +166,15 @@ __host__ __device__ __forceinline__ int hal_rule_lo(const hal_score_rule& r, int
 __device__ __forceinline__ float hal_rule_bias(const hal_score_rule& r, int head, int back) {
   return r.bias[(size_t)head * r.bias_len + (back < r.bias_len ? back : r.bias_len - 1)];
 }
-// 1 / (l + the sink's term) for sums taken relative to the maximum m
+// what a finished row's sums (taken relative to the maximum m) are multiplied by:
+// 1 / (l + the sink's term), or exp(m) for weights that are not normalised
 __device__ __forceinline__ float hal_rule_inverse(const hal_score_rule& r, float m, float l) {
-  return 1.0f / (r.sink ? l + expf(-m) : l);
+  if (r.sink == HAL_WEIGHTS_SIGMOID) return expf(m);
+  return 1.0f / (r.sink == HAL_WEIGHTS_SINK ? l + expf(-m) : l);
+}
+// ln sigmoid(s) = min(s, 0) - ln(1 + exp(-|s|))
+__device__ __forceinline__ float hal_log_sigmoid(float s) {
+  return fminf(s, 0.f) - log1pf(expf(-fabsf(s)));
 }
 
 // Sum over a block of up to 1024 threads; every thread gets the result.

@@ -404,3 +404,195 @@ extern "C" int hal_qk_norm_pack(const float* q, int ldq, const float* k, int ldk
   HAL_LAUNCH_CHECK();
   return 0;
 }
+
+// ---- several copies of the residual stream.  x [S][T][W] float32; a workgroup a row.
+// With y (a part's result, float32 [T][W]) every copy is made anew from the old ones,
+//   x_t <- sum_s mix[s][t] x_s + m * out[t] * y,
+// and, if `read`, the row that the next part reads is made of the new copies,
+//   u = sum_s in[s] x_s   (in null: every copy counts once),
+// and either written as it is (norm_w null) or normed: u / sqrt(mean(u^2) + eps) * (offset + w).
+// `rows` (or null): which rows of x the workgroups take; the results are written in that order.
+template <typename TO, int MAXS>
+__global__ void streams_step_kernel(float* __restrict__ x, size_t copy_stride, int S, const float* __restrict__ y,
+                                    const void* __restrict__ mix, const void* __restrict__ outw, float m,
+                                    const void* __restrict__ inw, int c_dtype, int read,
+                                    const void* __restrict__ norm_w, int norm_dtype, float offset, float eps,
+                                    TO* __restrict__ result, const int* __restrict__ rows, int W) {
+  extern __shared__ float u_row[];
+  __shared__ float scratch[16];
+  const size_t t = rows ? (size_t)rows[blockIdx.x] : (size_t)blockIdx.x;
+  float cm[MAXS][MAXS], co[MAXS], ci[MAXS];
+#pragma unroll
+  for (int s = 0; s < MAXS; ++s) {
+    co[s] = (y && s < S) ? m * load_as_f32(outw, c_dtype, s) : 0.f;
+    ci[s] = s < S ? (inw ? load_as_f32(inw, c_dtype, s) : 1.0f) : 0.f;
+#pragma unroll
+    for (int d = 0; d < MAXS; ++d) cm[s][d] = (y && s < S && d < S) ? load_as_f32(mix, c_dtype, s * S + d) : 0.f;
+  }
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < W; i += blockDim.x) {
+    float xs[MAXS];
+#pragma unroll
+    for (int s = 0; s < MAXS; ++s) xs[s] = s < S ? x[s * copy_stride + t * W + i] : 0.f;
+    if (y) {
+      const float yv = y[t * W + i];
+      float nx[MAXS];
+#pragma unroll
+      for (int d = 0; d < MAXS; ++d) {
+        float acc = co[d] * yv;
+#pragma unroll
+        for (int s = 0; s < MAXS; ++s) acc = fmaf(cm[s][d], xs[s], acc);
+        nx[d] = acc;
+      }
+#pragma unroll
+      for (int s = 0; s < MAXS; ++s) {
+        xs[s] = nx[s];
+        if (s < S) x[s * copy_stride + t * W + i] = nx[s];
+      }
+    }
+    if (read) {
+      float u = 0.f;
+#pragma unroll
+      for (int s = 0; s < MAXS; ++s) u = fmaf(ci[s], xs[s], u);
+      if (norm_w) {
+        u_row[i] = u;
+        ss += u * u;
+      } else {
+        result[(size_t)blockIdx.x * W + i] = from_f32<TO>(u);
+      }
+    }
+  }
+  if (!read || !norm_w) return;
+  const float total = block_sum(ss, scratch);
+  const float rstd = 1.0f / sqrtf(total / (float)W + eps);
+  for (int i = threadIdx.x; i < W; i += blockDim.x)  // (a thread reads back what it wrote itself)
+    result[(size_t)blockIdx.x * W + i] = from_f32<TO>(u_row[i] * rstd * (offset + load_as_f32(norm_w, norm_dtype, i)));
+}
+
+extern "C" int hal_streams_step(float* x, long long copy_stride, int S, const float* y, const void* mix,
+                                const void* outw, float m, const void* inw, int c_dtype, int read,
+                                const void* norm_w, int norm_dtype, float offset, float eps, void* result,
+                                int result_dtype, const int* rows, int n_rows, int W, hipStream_t stream) {
+  HAL_REQUIRE(S >= 1 && S <= 8, "hal_streams_step: %d copies of the stream (1 to 8)", S);
+  HAL_REQUIRE(n_rows >= 0 && W > 0 && W <= 16384, "hal_streams_step: bad sizes rows=%d width=%d", n_rows, W);
+  HAL_REQUIRE(y == nullptr || (mix && outw && rows == nullptr), "hal_streams_step: an update needs its weights and all rows");
+  HAL_REQUIRE(!read || result, "hal_streams_step: nowhere to write the row that was read");
+  HAL_REQUIRE(y || read, "hal_streams_step: nothing to do");
+  HAL_REQUIRE(result_dtype == HAL_F32 || result_dtype == HAL_BF16, "hal_streams_step: dtype %d", result_dtype);
+  if (n_rows == 0) return 0;
+  const size_t lds = (read && norm_w) ? (size_t)W * sizeof(float) : 0;
+#define STREAMS_LAUNCH(T_, M_)                                                                                      \
+  hipLaunchKernelGGL((streams_step_kernel<T_, M_>), dim3(n_rows), dim3(256), lds, stream, x, (size_t)copy_stride, S, y, \
+                     mix, outw, m, inw, c_dtype, read, norm_w, norm_dtype, offset, eps, (T_*)result, rows, W)
+#define STREAMS_BY_COUNT(T_)                \
+  do {                                      \
+    if (S <= 2) STREAMS_LAUNCH(T_, 2);      \
+    else if (S <= 4) STREAMS_LAUNCH(T_, 4); \
+    else STREAMS_LAUNCH(T_, 8);             \
+  } while (0)
+  if (result_dtype == HAL_F32) STREAMS_BY_COUNT(float);
+  else STREAMS_BY_COUNT(bf16_t);
+#undef STREAMS_BY_COUNT
+#undef STREAMS_LAUNCH
+  HAL_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---- every head of q, k and v divided by its own root mean square (no weight), packed as
+// [H heads of D | K heads of D | K heads of D] with zeros beyond a head's entries, keys and
+// values appended to the pages as well (k_pages null: not).  A wave a (token, head). ---------
+template <typename T>
+__global__ void head_norm_pack_kernel(const float* __restrict__ q, int ldq, const float* __restrict__ k, int ldk,
+                                      const float* __restrict__ v, int ldv, float eps,
+                                      const int* __restrict__ positions, T* __restrict__ out, int row_stride,
+                                      int n_tokens, int H, int K, int dq, int dv, int D,
+                                      const int* __restrict__ token_seg, const int* __restrict__ block_table,
+                                      int bt_stride, T* __restrict__ k_pages, T* __restrict__ v_pages, int page_size,
+                                      int n_pages, bool tiled) {
+  const int lane = threadIdx.x % HAL_WAVE, slots = H + 2 * K;
+  const size_t unit = (size_t)blockIdx.x * (blockDim.x / HAL_WAVE) + threadIdx.x / HAL_WAVE;
+  if (unit >= (size_t)n_tokens * slots) return;
+  const size_t t = unit / slots;
+  const int hs = (int)(unit % slots);
+  const int kind = hs < H ? 0 : (hs < H + K ? 1 : 2);
+  const int head = kind == 0 ? hs : (kind == 1 ? hs - H : hs - H - K);
+  const int n = kind == 2 ? dv : dq;
+  const float* src = kind == 0 ? q + t * ldq + (size_t)head * dq
+                               : (kind == 1 ? k + t * ldk + (size_t)head * dq : v + t * ldv + (size_t)head * dv);
+  float ss = 0.f;
+  for (int i = lane; i < n; i += HAL_WAVE) ss += src[i] * src[i];
+  const float rstd = 1.0f / sqrtf(wave_sum(ss) / (float)n + eps);
+  long long page = -1;
+  int off = 0;
+  if (k_pages && kind != 0) {
+    const int pos = positions[t];
+    page = block_table[(size_t)token_seg[t] * bt_stride + pos / page_size];
+    off = pos % page_size;
+    if (page < 0 || page >= n_pages) page = -1;  // checked on the host
+  }
+  T* o = out + t * row_stride + (size_t)hs * D;
+  for (int d = lane; d < D; d += HAL_WAVE) {
+    const T x = from_f32<T>(d < n ? src[d] * rstd : 0.f);
+    o[d] = x;
+    if (page >= 0) {
+      if (kind == 1) k_pages[((size_t)page * K + head) * page_size * D + kv_key_offset(tiled, page_size, D, off, d)] = x;
+      else v_pages[((size_t)page * K + head) * D * page_size + kv_value_offset(tiled, page_size, D, off, d)] = x;
+    }
+  }
+}
+
+extern "C" int hal_head_norm_pack(const float* q, int ldq, const float* k, int ldk, const float* v, int ldv, float eps,
+                                  const int* positions, void* out, int row_stride, int dtype, int n_tokens, int H,
+                                  int K, int dq, int dv, int D, const int* token_seg, const int* block_table,
+                                  int bt_stride, void* k_pages, void* v_pages, int page_size, int n_pages, int tiled,
+                                  hipStream_t stream) {
+  HAL_REQUIRE(k_pages == nullptr || (v_pages && token_seg && block_table && positions && page_size > 0 && n_pages > 0),
+              "hal_head_norm_pack: pages without the arrays that say where a token's key goes");
+  HAL_REQUIRE(n_tokens >= 0 && H > 0 && K > 0 && dq > 0 && dv > 0 && D >= dq && D >= dv,
+              "hal_head_norm_pack: bad sizes T=%d H=%d K=%d dq=%d dv=%d D=%d", n_tokens, H, K, dq, dv, D);
+  HAL_REQUIRE(row_stride >= (H + 2 * K) * D && ldq >= H * dq && ldk >= K * dq && ldv >= K * dv,
+              "hal_head_norm_pack: rows too short");
+  HAL_REQUIRE(dtype == HAL_F32 || dtype == HAL_BF16, "hal_head_norm_pack: dtype %d", dtype);
+  if (n_tokens == 0) return 0;
+  const long long units = (long long)n_tokens * (H + 2 * K);
+  const dim3 grid((unsigned)((units + 3) / 4));
+  if (dtype == HAL_F32)
+    hipLaunchKernelGGL(head_norm_pack_kernel<float>, grid, dim3(256), 0, stream, q, ldq, k, ldk, v, ldv, eps, positions,
+                       (float*)out, row_stride, n_tokens, H, K, dq, dv, D, token_seg, block_table, bt_stride,
+                       (float*)k_pages, (float*)v_pages, page_size, n_pages, tiled != 0);
+  else
+    hipLaunchKernelGGL(head_norm_pack_kernel<bf16_t>, grid, dim3(256), 0, stream, q, ldq, k, ldk, v, ldv, eps, positions,
+                       (bf16_t*)out, row_stride, n_tokens, H, K, dq, dv, D, token_seg, block_table, bt_stride,
+                       (bf16_t*)k_pages, (bf16_t*)v_pages, page_size, n_pages, tiled != 0);
+  HAL_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---- y[t, h * n + j] = x[t, h * x_head + j] * sigmoid(g[t, h]) for j < n: every head's result
+// times one number of its own, the heads' padding dropped on the way -------------------------
+template <typename T>
+__global__ void head_gate_cols_kernel(const T* __restrict__ x, int ldx, int x_head, const float* __restrict__ g, int ldg,
+                                      T* __restrict__ y, int n, int H) {
+  const size_t t = blockIdx.x;
+  for (int e = threadIdx.x; e < H * n; e += blockDim.x) {
+    const int h = e / n, j = e % n;
+    const float gate = 1.0f / (1.0f + expf(-g[t * ldg + h]));
+    y[t * H * n + e] = from_f32<T>(to_f32(x[t * ldx + (size_t)h * x_head + j]) * gate);
+  }
+}
+
+extern "C" int hal_head_gate_cols(const void* x, int ldx, int x_head, const float* g, int ldg, void* y, int n, int H,
+                                  int dtype, int n_tokens, hipStream_t stream) {
+  HAL_REQUIRE(n_tokens >= 0 && H > 0 && n > 0 && x_head >= n && ldx >= H * x_head && ldg >= H,
+              "hal_head_gate_cols: bad sizes T=%d heads=%d n=%d of %d", n_tokens, H, n, x_head);
+  HAL_REQUIRE(dtype == HAL_F32 || dtype == HAL_BF16, "hal_head_gate_cols: dtype %d", dtype);
+  if (n_tokens == 0) return 0;
+  if (dtype == HAL_F32)
+    hipLaunchKernelGGL(head_gate_cols_kernel<float>, dim3(n_tokens), dim3(256), 0, stream, (const float*)x, ldx, x_head,
+                       g, ldg, (float*)y, n, H);
+  else
+    hipLaunchKernelGGL(head_gate_cols_kernel<bf16_t>, dim3(n_tokens), dim3(256), 0, stream, (const bf16_t*)x, ldx, x_head,
+                       g, ldg, (bf16_t*)y, n, H);
+  HAL_LAUNCH_CHECK();
+  return 0;
+}

@@ -421,7 +421,7 @@ def attention_mfma(q, q_row_stride, plan_dev, ctx, group, kv, n_heads, scale, wi
         P(group.block_table), group.block_table.shape[1], P(kv.k), P(kv.v), P(part_o), P(part_ml),
         P(counters), N_COUNTERS, n_heads, n_kv, head_dim, page_size, 1 if getattr(kv, "tiled", False) else 0,
         ctypes.c_float(scale), window, rule.chunk, P(bias), 0 if bias is None else bias.shape[1],
-        1 if rule.sink else 0, plan.max_parts, ops._stream(),
+        rule.weights_code(), plan.max_parts, ops._stream(),
     )
     ops._check(lib, rc)
     return out

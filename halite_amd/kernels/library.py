@@ -47,6 +47,7 @@ CORE_SOURCES = [
     "latent_moe.hip",
     "stream_ops.hip",
     "recurrent.hip",
+    "delta_rule.hip",
 ]
 ATTENTION_SOURCES = ["runtime.hip", "attention_mfma.hip"]
 

@@ -30,16 +30,25 @@ class ScoreRule:
     start of its own chunk of that many positions (counted from position 0 of the
     request).  ``bias``: float32 ``[heads, distances]`` on the device, added to the scaled
     score of the key ``n`` tokens back at ``[head, min(n, distances - 1)]``.  ``sink``: the
-    softmax has one more term of score 0 that carries no value."""
+    softmax has one more term of score 0 that carries no value.  ``sigmoid``: no softmax: a
+    visible key's weight is the sigmoid of its score (scaled, with the bias), and the weights
+    are not normalised over the keys."""
 
     chunk: int = 0
     bias: torch.Tensor | None = None
     sink: bool = False
     # the same table times log2 e, for the kernel whose exponentials are to the base 2
     bias_log2: torch.Tensor | None = None
+    sigmoid: bool = False
 
     def plain(self) -> bool:
-        return self.chunk == 0 and self.bias is None and not self.sink
+        return self.chunk == 0 and self.bias is None and not self.sink and not self.sigmoid
+
+    def weights_code(self) -> int:
+        """The kernels' number for how a row's weights are made (``HAL_WEIGHTS_*``)."""
+        if self.sigmoid and self.sink:
+            raise KernelError("a sink belongs to a softmax; sigmoid weights have none")
+        return 2 if self.sigmoid else (1 if self.sink else 0)
 
 
 @dataclass
@@ -384,7 +393,7 @@ def attention_simple(
             _ptr(positions), _ptr(token_seg), _ptr(block_table), block_table.shape[1],
             _ptr(k_pages), _ptr(v_pages), _ptr(part), n, n_heads, n_kv, head_dim, page_size, n_pages,
             ctypes.c_float(scale), window, rule.chunk, _ptr(bias), 0 if bias is None else bias.shape[1],
-            1 if rule.sink else 0, max_kv_len, min_q_len, _stream(),
+            rule.weights_code(), max_kv_len, min_q_len, _stream(),
         ),
     )
     return out
@@ -759,7 +768,7 @@ def grouped_gemm(
     w_up: torch.Tensor | None = None, limit: float = 0.0, alpha: float = 0.0,
     group_offsets: torch.Tensor | None = None, tile_offsets: torch.Tensor | None = None,
     row_src: torch.Tensor | None = None, src_div: int = 1, row_dst: torch.Tensor | None = None,
-    gate: torch.Tensor | None = None, add: bool = False, mfma: bool = True,
+    gate: torch.Tensor | None = None, add: bool = False, mfma: bool = True, relu_squared: bool = False,
 ) -> torch.Tensor:
     """``y_g = x_g @ w[g].T`` for every group ``g`` of ``w`` ``[G, N, K]`` in one launch
     (float32 accumulation).  Heads: every group has all ``n_rows`` rows; group ``g`` reads
@@ -769,7 +778,8 @@ def grouped_gemm(
     ``group_offsets`` / ``tile_offsets`` (from ``moe_sort``) cut a list of ``n_rows`` rows
     into the groups' slices; row ``i`` reads ``x[row_src[i] // src_div]`` and writes
     ``y[row_dst[i]]`` (``i`` without the arrays); with ``w_up`` the result is the clamped
-    gated activation of the two products.  ``add``: added into a float32 ``y``."""
+    gated activation of the two products; without it and with ``relu_squared`` the square of
+    the product's positive part.  ``add``: added into a float32 ``y``."""
     lib = library.core_library()
     _dev(w, w_up, group_offsets, tile_offsets, row_src, row_dst)
     for t in (x, y, gate):
@@ -778,6 +788,7 @@ def grouped_gemm(
     _need(w.dim() == 3 and w.dtype == x.dtype and (w_up is None or (w_up.shape == w.shape and w_up.dtype == w.dtype)),
           "grouped_gemm: weights [G, N, K] of the rows' element type")
     g, n, k = w.shape
+    _need(not relu_squared or w_up is None, "grouped_gemm: the square of relu is for a product without a gate")
     _need(gate is None or gate.dtype == torch.float32, "grouped_gemm: a float32 gate")
     _need(not add or y.dtype == torch.float32, "grouped_gemm: only a float32 result is added into")
     if group_offsets is None:
@@ -798,7 +809,7 @@ def grouped_gemm(
         dtype_code(x.dtype), _ptr(y), y.stride(0), y_group_cols, y_col0, dtype_code(y.dtype), 1 if add else 0,
         n_rows, n, k, g, _ptr(group_offsets), _ptr(tile_offsets), _ptr(row_src), src_div, _ptr(row_dst),
         _ptr(gate), 0 if gate is None else gate.stride(0), ctypes.c_float(limit), ctypes.c_float(alpha),
-        1 if mfma else 0, _stream()))
+        1 if relu_squared else 0, 1 if mfma else 0, _stream()))
     return y
 
 
@@ -1081,3 +1092,142 @@ def gated_part_norm(y: torch.Tensor, z: torch.Tensor, weight: torch.Tensor, eps:
     _check(lib, lib.hal_gated_part_norm(_ptr(y), _ptr(z), z.stride(0), _ptr(weight), dtype_code(weight.dtype),
                                         ctypes.c_float(eps), _ptr(out), dtype_code(out_dtype), n, inner, parts, _stream()))
     return out
+
+
+# -- the generalized delta rule; copies of the stream; per-head norms and gates -------------------
+
+
+def delta_rule(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, a_raw: torch.Tensor, x1: torch.Tensor,
+               w2: torch.Tensor, w0: torch.Tensor, a_bias: torch.Tensor, state: torch.Tensor,
+               seg_q_start: torch.Tensor, seg_q_len: torch.Tensor, token_slot: torch.Tensor,
+               decay_rate: float, unit_eps: float) -> torch.Tensor:
+    """The generalized delta rule over every request's tokens of the step: per head
+    ``S <- diag(w) S - (a * u)(u^T S) + k v^T``, ``o = S^T r`` with ``w = exp(-decay_rate *
+    sigmoid(w0 + W2 tanh(x1)))``, ``a = sigmoid(a_raw + a_bias)`` and the unit key ``u = k /
+    sqrt(sum(k^2) + unit_eps)``.  ``r``, ``k``, ``v``, ``a_raw``: float32 ``[T, heads * dim]``
+    (row-strided views allowed); ``x1`` float32 ``[T, rank]``; ``state`` float32 ``[slots,
+    heads, dim, dim]`` (key channel, value channel), read and left as the step's last state.
+    Returns float32 ``[T, heads * dim]``."""
+    lib = library.core_library()
+    _, heads, d, d2 = state.shape
+    n, inner = r.shape[0], heads * d
+    for t, what in ((r, "r"), (k, "k"), (v, "v"), (a_raw, "a")):
+        _rows_f32(t, inner, f"delta_rule {what}")
+        _need(t.shape[0] == n, "delta_rule: one row a token")
+    lora = x1.shape[1]
+    _rows_f32(x1, lora, "delta_rule x1")
+    _dev(w2, w0, a_bias, state, seg_q_start, seg_q_len, token_slot)
+    _i32(seg_q_start, "seg_q_start"), _i32(seg_q_len, "seg_q_len"), _i32(token_slot, "token_slot")
+    _need(state.dtype == torch.float32 and d == d2, "delta_rule: a float32 state [slots, heads, dim, dim]")
+    _need(w2.shape == (inner, lora) and w0.numel() == inner and a_bias.numel() == inner
+          and w2.dtype == w0.dtype == a_bias.dtype, "delta_rule: w2 [heads * dim, rank], w0 and a_bias [heads * dim] of one type")
+    _need(token_slot.numel() == n and seg_q_start.numel() == seg_q_len.numel(), "delta_rule: the step's arrays")
+    dp = 16 if d <= 16 else 32 if d <= 32 else 64 if d <= 64 else 128 if d <= 128 else 256
+    pre = torch.empty((n, heads, 5, dp), dtype=torch.float32, device=r.device)
+    o = torch.empty((n, inner), dtype=torch.float32, device=r.device)
+    _check(lib, lib.hal_delta_rule(
+        _ptr(r), r.stride(0), _ptr(k), k.stride(0), _ptr(v), v.stride(0), _ptr(a_raw), a_raw.stride(0),
+        _ptr(x1), x1.stride(0), _ptr(w2), _ptr(w0), _ptr(a_bias), dtype_code(w2.dtype), lora,
+        ctypes.c_float(decay_rate), ctypes.c_float(unit_eps), _ptr(pre), _ptr(state), _ptr(seg_q_start),
+        _ptr(seg_q_len), _ptr(token_slot), _ptr(o), n, seg_q_start.numel(), heads, d, _stream()))
+    return o
+
+
+def head_norm_gate(y: torch.Tensor, z: torch.Tensor | None, weight: torch.Tensor | None, eps: float, heads: int,
+                   out_dtype: torch.dtype) -> torch.Tensor:
+    """Every head of the float32 rows ``y`` ``[T, heads * dim]`` divided by its own root mean
+    square, times ``weight`` (of the row's length) and ``sigmoid(z)`` (float32, a row-strided
+    view is allowed)."""
+    lib = library.core_library()
+    _dev(y, weight)
+    n, inner = y.shape
+    _need(y.dtype == torch.float32 and inner % heads == 0, "head_norm_gate: float32 rows of whole heads")
+    if z is not None:
+        _rows_f32(z, inner, "head_norm_gate z")
+    _need(weight is None or weight.numel() == inner, "head_norm_gate: a weight of the row's length")
+    out = torch.empty((n, inner), dtype=out_dtype, device=y.device)
+    _check(lib, lib.hal_head_norm_gate(_ptr(y), _ptr(z), 0 if z is None else z.stride(0), _ptr(weight),
+                                       dtype_code(weight.dtype) if weight is not None else F32, ctypes.c_float(eps),
+                                       _ptr(out), dtype_code(out_dtype), n, heads, inner // heads, _stream()))
+    return out
+
+
+def streams_step(x: torch.Tensor, *, y: torch.Tensor | None = None, mix: torch.Tensor | None = None,
+                 out: torch.Tensor | None = None, mult: float = 1.0, read: bool = False,
+                 inw: torch.Tensor | None = None, norm_weight: torch.Tensor | None = None, offset: float = 0.0,
+                 eps: float = 0.0, dtype: torch.dtype = torch.float32, rows: torch.Tensor | None = None):
+    """One pass over the copies ``x`` (float32 ``[S, T, W]``) of the residual stream.  With
+    ``y`` (float32 ``[T, W]``) every copy is made anew from the old ones, ``x_t <- sum_s
+    mix[s, t] x_s + mult * out[t] * y``.  With ``read`` the row ``u = sum_s inw[s] x_s``
+    (``inw`` None: the plain sum) of the new copies comes back, as it is (float32) or, with
+    ``norm_weight``, as ``u / sqrt(mean(u^2) + eps) * (offset + norm_weight)`` in ``dtype``;
+    ``rows`` (only without ``y``): of those rows alone."""
+    lib = library.core_library()
+    _dev(x, y, mix, out, inw, norm_weight, rows)
+    _i32(rows, "rows")
+    _need(x.dtype == torch.float32 and x.dim() == 3, "streams_step: float32 copies [S, T, W]")
+    s, t, w = x.shape
+    _need(y is None or (y.dtype == torch.float32 and y.shape == (t, w) and mix is not None and out is not None
+                        and mix.shape == (s, s) and out.numel() == s and mix.dtype == out.dtype and rows is None),
+          "streams_step: an update takes float32 y [T, W], mix [S, S] and out [S] of one type, and all rows")
+    _need(inw is None or (inw.numel() == s and (mix is None or inw.dtype == mix.dtype)), "streams_step: inw [S]")
+    _need(norm_weight is None or norm_weight.numel() == w, "streams_step: a norm weight of the rows' width")
+    c_dtype = mix.dtype if mix is not None else (inw.dtype if inw is not None else torch.float32)
+    n = t if rows is None else rows.numel()
+    result = None
+    if read:
+        result = torch.empty((n, w), dtype=dtype if norm_weight is not None else torch.float32, device=x.device)
+    _check(lib, lib.hal_streams_step(
+        _ptr(x), ctypes.c_longlong(t * w), s, _ptr(y), _ptr(mix), _ptr(out), ctypes.c_float(mult), _ptr(inw),
+        dtype_code(c_dtype), 1 if read else 0, _ptr(norm_weight),
+        dtype_code(norm_weight.dtype) if norm_weight is not None else F32, ctypes.c_float(offset), ctypes.c_float(eps),
+        _ptr(result), dtype_code(result.dtype) if result is not None else F32, _ptr(rows), n, w, _stream()))
+    return result
+
+
+def head_norm_pack(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, eps: float, n_heads: int, n_kv_heads: int,
+                   qk_dim: int, v_dim: int, head_dim: int, out_dtype: torch.dtype,
+                   positions: torch.Tensor | None = None, token_seg: torch.Tensor | None = None,
+                   block_table: torch.Tensor | None = None, k_pages: torch.Tensor | None = None,
+                   v_pages: torch.Tensor | None = None, page_size: int = 0, tiled: bool = False) -> torch.Tensor:
+    """From float32 projections (row-strided views allowed): every head of ``q``, ``k`` and
+    ``v`` divided by its own root mean square (no weight); the packed rows ``[q heads | k heads
+    | v heads]`` of ``head_dim`` entries a head (zero beyond ``qk_dim`` / ``v_dim``) come back.
+    With ``k_pages`` and ``v_pages`` keys and values are appended to the pages as well."""
+    lib = library.core_library()
+    n = q.shape[0]
+    _rows_f32(q, n_heads * qk_dim, "head_norm_pack q"), _rows_f32(k, n_kv_heads * qk_dim, "head_norm_pack k")
+    _rows_f32(v, n_kv_heads * v_dim, "head_norm_pack v")
+    _need(head_dim >= max(qk_dim, v_dim), "head_norm_pack: head sizes")
+    out = torch.empty((n, (n_heads + 2 * n_kv_heads) * head_dim), dtype=out_dtype, device=q.device)
+    n_pages = 0
+    if k_pages is not None:
+        _dev(positions, token_seg, block_table, k_pages, v_pages)
+        _i32(positions, "positions"), _i32(token_seg, "token_seg"), _i32(block_table, "block_table")
+        n_pages = k_pages.shape[0]
+        _need(v_pages is not None and k_pages.dtype == out_dtype and v_pages.dtype == out_dtype
+              and k_pages.shape == (n_pages, n_kv_heads, page_size, head_dim)
+              and v_pages.shape == (n_pages, n_kv_heads, head_dim, page_size), "head_norm_pack: page shapes")
+        _need(positions is not None and positions.numel() == n and token_seg is not None and token_seg.numel() == n
+              and block_table is not None and block_table.dim() == 2, "head_norm_pack: the step's arrays")
+    _check(lib, lib.hal_head_norm_pack(
+        _ptr(q), q.stride(0), _ptr(k), k.stride(0), _ptr(v), v.stride(0), ctypes.c_float(eps), _ptr(positions),
+        _ptr(out), out.shape[1], dtype_code(out_dtype), n, n_heads, n_kv_heads, qk_dim, v_dim, head_dim,
+        _ptr(token_seg), _ptr(block_table), 0 if block_table is None else block_table.shape[1],
+        _ptr(k_pages), _ptr(v_pages), page_size, n_pages, 1 if tiled else 0, _stream()))
+    return out
+
+
+def head_gate_cols(x: torch.Tensor, x_head: int, gate: torch.Tensor, n: int, n_heads: int) -> torch.Tensor:
+    """``y[t, h * n + j] = x[t, h * x_head + j] * sigmoid(gate[t, h])`` for ``j < n``: every
+    head's first ``n`` entries times a number of the head's own (``gate`` float32, a
+    row-strided view is allowed)."""
+    lib = library.core_library()
+    _dev(x)
+    _need(x.dim() == 2 and x.shape[1] >= n_heads * x_head and x_head >= n, "head_gate_cols: rows of padded heads")
+    _rows_f32(gate, n_heads, "head_gate_cols gate")
+    _need(gate.shape[0] == x.shape[0], "head_gate_cols: one gate row a token")
+    y = torch.empty((x.shape[0], n_heads * n), dtype=x.dtype, device=x.device)
+    _check(lib, lib.hal_head_gate_cols(_ptr(x), x.shape[1], x_head, _ptr(gate), gate.stride(0), _ptr(y), n, n_heads,
+                                       dtype_code(x.dtype), x.shape[0], _stream()))
+    return y

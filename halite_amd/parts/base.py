@@ -242,7 +242,28 @@ class RotaryPositionEncoding(PositionEncoding):
 
 
 class Embedding(Part):
-    def forward(self, tokens: torch.Tensor) -> torch.Tensor:
+    def forward(self, tokens: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+        """The tokens' rows as float32 ``[T, width]``, written to ``out`` if that is given."""
+        raise NotImplementedError
+
+
+class Connection(Part):
+    """How a part's input is read from the residual stream and how its result gets back
+    there, for arrangements that keep the stream in ``copies`` copies ``[copies, T, width]``."""
+
+    @property
+    def copies(self) -> int:
+        raise NotImplementedError
+
+    def step(self, x: torch.Tensor, pending, norm: "Norm") -> torch.Tensor:
+        """Writes what is ``pending`` (None, or ``(y, connection)``: a part's float32 result
+        and the connection it goes back through) into the copies ``x``, then returns the
+        rows that the next part reads through this connection, normed by ``norm``."""
+        raise NotImplementedError
+
+    def leave(self, x: torch.Tensor, pending, rows: torch.Tensor | None) -> torch.Tensor:
+        """Writes what is ``pending`` and returns the model's one stream (float32; of
+        ``rows`` alone if given)."""
         raise NotImplementedError
 
 
@@ -285,6 +306,7 @@ FEED_FORWARDS = Registry("feed-forward")
 NORMS = Registry("norm")
 POSITIONS = Registry("position encoding")
 EMBEDDINGS = Registry("embedding")
+CONNECTIONS = Registry("connection")
 HEADS = Registry("head")
 class Arrangement:
     """The order in which a layer's parts act on the residual stream.

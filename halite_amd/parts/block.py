@@ -13,7 +13,7 @@ from __future__ import annotations
 import torch
 
 from ..kernels import ops
-from .base import FEED_FORWARDS, MIXERS, NORMS, Arrangement, register_arrangement
+from .base import CONNECTIONS, FEED_FORWARDS, MIXERS, NORMS, Arrangement, register_arrangement
 from .norm import RMSNorm
 
 
@@ -158,3 +158,46 @@ class PostNormBlock(Arrangement):
         if dtype != torch.float32:
             ctx.rounded_rows = (run.index, x)
         return None
+
+
+@register_arrangement("hyper_pre_norm")
+class HyperPreNormBlock(Arrangement):
+    """A pre-norm block on a residual stream that is kept in copies: each of the two parts
+    reads its input through a connection of its own (``mixer_link``, ``ff_link``), which also
+    says how the part's result gets back into the copies.  A layer may leave the
+    feed-forward (with its norm and connection) out.
+
+    The stream handed from block to block is ``[copies, T, width]`` float32.  A part's
+    result is left pending, with its connection, for whoever reads next: the write of one
+    part and the read and norm of the next are one pass over the copies."""
+
+    graph_safe = True
+    roles = {"mixer_norm": NORMS, "mixer": MIXERS, "mixer_link": CONNECTIONS,
+             "ff_norm": NORMS, "ff": FEED_FORWARDS, "ff_link": CONNECTIONS}
+    optional = ("ff_norm", "ff", "ff_link")
+
+    def __init__(self, parts):
+        super().__init__(parts)
+        self.mixer_norm, self.mixer_link = parts["mixer_norm"], parts["mixer_link"]
+        self.ff_norm, self.ff, self.ff_link = parts.get("ff_norm"), parts.get("ff"), parts.get("ff_link")
+        if len({self.ff is None, self.ff_norm is None, self.ff_link is None}) != 1:
+            raise ValueError("a block has a feed-forward with its norm and connection, or none of them")
+        if self.ff_link is not None and self.ff_link.copies != self.mixer_link.copies:
+            raise ValueError("a block's connections keep different numbers of copies")
+
+    @property
+    def stream_copies(self) -> int:
+        return self.mixer_link.copies
+
+    def forward(self, h, pending, ctx, run):
+        x = self.mixer_link.step(h, pending, self.mixer_norm)
+        pending = (self.mixer.forward(x, ctx, run), self.mixer_link)
+        if self.ff is not None:
+            x = self.ff_link.step(h, pending, self.ff_norm)
+            pending = (self.ff.forward(x, ctx), self.ff_link)
+        return pending
+
+    def leave(self, h, pending, rows):
+        """The model's one stream after the last block (of ``rows`` alone if given)."""
+        link = pending[1] if pending is not None else self.mixer_link
+        return link.leave(h, pending, rows)

@@ -39,8 +39,8 @@ class Decoder:
     def __init__(self, spec: ModelSpec, dtype: torch.dtype, device: torch.device | str,
                  tiled_weights: bool = False):
         # the kinds of parts register themselves when their modules are imported
-        from . import (attention, block, embedding, feedforward, latent_attention, mixer_sum, moe, norm,  # noqa: F401
-                       normed_attention, rope, state_space)
+        from . import (attention, block, connection, embedding, feedforward, general_delta, latent_attention,  # noqa: F401
+                       mixer_sum, moe, norm, normed_attention, rope, sigmoid_attention, state_space)
 
         self.spec = spec
         self.dtype = dtype
@@ -63,6 +63,12 @@ class Decoder:
         self.runs = [
             RunBinding(index=i, appends=run.cache_from is None) for i, run in enumerate(spec.order)
         ]
+        # an arrangement may keep the residual stream in several copies ([copies, T, width]);
+        # then every block of the model does, and the last one says how they become one again
+        copies = {getattr(self.layers[run.layer], "stream_copies", None) for run in spec.order}
+        if len(copies) != 1:
+            raise ConfigError(f"the model's blocks keep the residual stream in different ways: {sorted(map(str, copies))} copies")
+        self.stream_copies = copies.pop()
 
     # -- declarations -------------------------------------------------------------
     def named_parts(self) -> dict[str, Part]:
@@ -104,7 +110,13 @@ class Decoder:
     def forward(self, ctx) -> torch.Tensor:
         """float32 logits ``[len(ctx.logit_rows), vocab]``; keys and values of all
         the step's tokens are in the cache afterwards."""
-        h = self.embedding.forward(ctx.tokens)
+        if self.stream_copies is None:
+            h = self.embedding.forward(ctx.tokens)
+        else:  # every copy starts as the embedding's output
+            h = torch.empty((self.stream_copies, ctx.tokens.numel(), self.spec.hidden_size), dtype=torch.float32,
+                            device=self.device)
+            for copy in h:
+                self.embedding.forward(ctx.tokens, out=copy)
         pending = None
         blocks = [self.layers[self.spec.order[run.index].layer] for run in self.runs]
         for i, run in enumerate(self.runs):
@@ -121,5 +133,8 @@ class Decoder:
                 pending = blocks[i].forward(h, pending, ctx, run)
         if ctx.n_logit_rows == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.device)
-        x = self.final_norm.forward(h, delta=pending, rows=ctx.logit_rows)
+        if self.stream_copies is not None:
+            x = self.final_norm.forward(blocks[-1].leave(h, pending, ctx.logit_rows))
+        else:
+            x = self.final_norm.forward(h, delta=pending, rows=ctx.logit_rows)
         return self.head.forward(x)

@@ -28,8 +28,8 @@ class TokenEmbedding(Embedding):
     def param_decls(self):
         return {"weight": ParamDecl((self.p.vocab_size, self.p.size))}
 
-    def forward(self, tokens):
-        return ops.embedding(tokens, self.weight, scale=self.p.scale)
+    def forward(self, tokens, out=None):
+        return ops.embedding(tokens, self.weight, out=out, scale=self.p.scale)
 
 
 class LinearHeadParams(BaseModel):

@@ -5,7 +5,7 @@ from __future__ import annotations
 import torch
 from typing import Literal
 
-from pydantic import BaseModel, Field, StrictInt, field_validator
+from pydantic import BaseModel, Field, StrictBool, StrictInt, field_validator
 
 from ..kernels import ops
 from .base import FEED_FORWARDS, FeedForward, ParamDecl
@@ -15,6 +15,9 @@ class GatedParams(BaseModel):
     hidden_size: StrictInt = Field(gt=0)
     intermediate_size: StrictInt = Field(gt=0)
     activation: str = "silu"
+    float32_result: StrictBool = False
+    """True: the last product's float32 sums come back unrounded (for an arrangement that
+    adds them into the float32 stream itself)."""
 
     @field_validator("activation")
     @classmethod
@@ -70,6 +73,8 @@ class GatedFeedForward(FeedForward):
     def forward(self, x, ctx, then=None):
         f = self.p.intermediate_size
         w = self.w_gate_up
+        if self.p.float32_result:
+            return self._forward_float32_result(x)
         # The gated product with SiLU·mul in its epilogue beats the library product and a
         # kernel for SiLU·mul up to 16 rows, and at 17 to 32 rows on matrices of up to 64 M
         # elements (measured in captured graphs: 50 against 56 us at 14336 x 4096, 23 against
@@ -97,6 +102,16 @@ class GatedFeedForward(FeedForward):
         else:
             act = ops.silu_mul(ops.linear(x, w))
         return ops.linear(act, self.w_out, tiled=self.t_out, next_norm=then)
+
+
+    def _forward_float32_result(self, x):
+        f = self.p.intermediate_size
+        m, d = x.shape
+        if self.t_gate is not None and x.dtype == torch.bfloat16 and d % 8 == 0 and m <= ops.SKINNY_ROWS:
+            act = ops.gemm_bf16_skinny(x, self.t_gate, w_up=self.t_up, tiled_shape=(f, d))
+        else:
+            act = ops.silu_mul(ops.linear(x, self.w_gate_up))
+        return ops.linear(act, self.w_out, out_dtype=torch.float32, tiled=self.t_out)
 
 
 class DenseParams(BaseModel):

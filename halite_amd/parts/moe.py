@@ -29,21 +29,32 @@ class ClampedGate(BaseModel):
     alpha: float = 1.702
 
 
+class SquaredRelu(BaseModel):
+    """An expert without a gate: ``W_down relu(W_up x)^2``."""
+
+    kind: Literal["relu_squared"]
+    intermediate_size: StrictInt = Field(gt=0)
+
+
 class MoEParams(BaseModel):
     hidden_size: StrictInt = Field(gt=0)
     n_experts: StrictInt = Field(gt=0)
     top_k: StrictInt = Field(gt=0)
-    expert: ClampedGate
+    expert: ClampedGate | SquaredRelu
     shared: ClampedGate | None = None
     score: Literal["sigmoid", "softmax"] = "sigmoid"
     normalize: StrictBool = True
     """The chosen scores are divided by their sum (+ ``norm_eps``)."""
     norm_eps: float = 1e-20
+    float32_result: StrictBool = False
+    """True: without a stream to add into, the float32 sum comes back unrounded."""
 
     @model_validator(mode="after")
     def _check(self):
         if self.top_k > self.n_experts:
             raise ValueError(f"top_k {self.top_k} of {self.n_experts} experts")
+        if self.shared is not None and isinstance(self.expert, SquaredRelu):
+            raise ValueError("a shared expert comes with gated experts")
         return self
 
 
@@ -53,12 +64,17 @@ class MixtureOfExperts(FeedForward):
     graph_safe = True
     adds_to_stream = True
 
+    @property
+    def gated(self) -> bool:
+        return isinstance(self.p.expert, ClampedGate)
+
     def param_decls(self):
         p = self.p
         d, f = p.hidden_size, p.expert.intermediate_size
         decls = {"router.weight": ParamDecl((p.n_experts, d))}
         for e in range(p.n_experts):
-            decls[f"experts.{e}.gate.weight"] = ParamDecl((f, d))
+            if self.gated:
+                decls[f"experts.{e}.gate.weight"] = ParamDecl((f, d))
             decls[f"experts.{e}.up.weight"] = ParamDecl((f, d))
             decls[f"experts.{e}.down.weight"] = ParamDecl((d, f))
         if p.shared is not None:
@@ -76,13 +92,14 @@ class MixtureOfExperts(FeedForward):
             raise ValueError("the experts' weights are stored with different element types")
         dt = kinds.pop()
         # all experts in one tensor per projection: the grouped products index them by expert
-        self.w_gate = torch.empty((n, f, d), dtype=dt, device=dev)
+        self.w_gate = torch.empty((n, f, d), dtype=dt, device=dev) if self.gated else None
         self.w_up = torch.empty((n, f, d), dtype=dt, device=dev)
         self.w_down = torch.empty((n, d, f), dtype=dt, device=dev)
         self.w_router = torch.empty((n, d), dtype=dtypes["router.weight"], device=dev)
         out = {"router.weight": self.w_router}
         for e in range(n):
-            out[f"experts.{e}.gate.weight"] = self.w_gate[e]
+            if self.gated:
+                out[f"experts.{e}.gate.weight"] = self.w_gate[e]
             out[f"experts.{e}.up.weight"] = self.w_up[e]
             out[f"experts.{e}.down.weight"] = self.w_down[e]
         if p.shared is not None:
@@ -110,8 +127,12 @@ class MixtureOfExperts(FeedForward):
         pairs = n * p.top_k
         # rows in the sorted order: row i belongs to pair order[i] = token * top_k + choice
         act = torch.empty((pairs, p.expert.intermediate_size), dtype=x.dtype, device=x.device)
-        ops.grouped_gemm(x, self.w_gate, act, n_rows=pairs, w_up=self.w_up, limit=p.expert.limit, alpha=p.expert.alpha,
-                         group_offsets=offsets, tile_offsets=tiles, row_src=order, src_div=p.top_k)
+        if self.gated:
+            ops.grouped_gemm(x, self.w_gate, act, n_rows=pairs, w_up=self.w_up, limit=p.expert.limit, alpha=p.expert.alpha,
+                             group_offsets=offsets, tile_offsets=tiles, row_src=order, src_div=p.top_k)
+        else:
+            ops.grouped_gemm(x, self.w_up, act, n_rows=pairs, relu_squared=True,
+                             group_offsets=offsets, tile_offsets=tiles, row_src=order, src_div=p.top_k)
         y = torch.empty((pairs, d), dtype=torch.float32, device=x.device)
         ops.grouped_gemm(act, self.w_down, y, n_rows=pairs, group_offsets=offsets, tile_offsets=tiles, row_dst=order)
         if p.shared is not None:
@@ -126,4 +147,6 @@ class MixtureOfExperts(FeedForward):
             # the shared expert's result rides along with the weighted sum
             extra = ops.linear(acts, self.ws_down, out_dtype=torch.float32, tiled=self.t_shared_down)
         ops.moe_combine(h, y, wgt, extra if p.shared is not None else None)
-        return None if add_to is not None else h.to(x.dtype)
+        if add_to is not None:
+            return None
+        return h if p.float32_result else h.to(x.dtype)

@@ -3,7 +3,7 @@
 from __future__ import annotations
 
 import torch
-from pydantic import BaseModel, Field, StrictBool, StrictInt
+from pydantic import BaseModel, Field, StrictBool, StrictInt, model_validator
 
 from ..kernels import ops
 from .base import NORMS, Norm, ParamDecl
@@ -16,6 +16,15 @@ class RMSNormParams(BaseModel):
     """True: the normalised value is rounded to the activation type before the weight
     multiplies it (the reference's order).  False: ``x * rstd * w`` in float32 and one
     rounding at the end."""
+    weight_offset: float = 0.0
+    """The stored weight is the multiplier's distance from this: the norm multiplies by
+    ``weight_offset + weight`` (float32; only in the unrounded order)."""
+
+    @model_validator(mode="after")
+    def _check(self):
+        if self.weight_offset != 0.0 and self.round_before_weight:
+            raise ValueError("a weight stored as a distance is added up in float32: round_before_weight must be false")
+        return self
 
 
 @NORMS.register("rmsnorm")
@@ -35,6 +44,9 @@ class RMSNorm(Norm):
         if not self.p.round_before_weight:
             if delta is not None:
                 ops.residual_add(h, delta)
+            if self.p.weight_offset != 0.0:
+                return ops.streams_step(h.view(1, *h.shape), read=True, norm_weight=self.weight, offset=self.p.weight_offset,
+                                        eps=self.p.eps, dtype=self.build.dtype, rows=rows)
             return ops.rmsnorm_exact(h, self.weight, self.p.eps, self.build.dtype, rows=rows)
         if isinstance(delta, ops.NormedRows):
             # the product before has added its result into h and prepared these rows
