@@ -147,7 +147,7 @@ def test_a_layer_names_the_parts_its_arrangement_has():
         Decoder(short, torch.float32, "cpu")
     other = spec.model_copy(deep=True)
     other.layers["0"].arrangement = "sandwich"
-    with pytest.raises(ConfigError, match="unknown arrangement 'sandwich'; known: parallel, post_norm, pre_norm"):
+    with pytest.raises(ConfigError, match="unknown arrangement 'sandwich'; known: hyper_pre_norm, parallel, post_norm, pre_norm"):
         Decoder(other, torch.float32, "cpu")
     # the keyword form and the dict form are the same description
     from halite_amd.config import LayerSpec
