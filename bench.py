@@ -100,8 +100,9 @@ class Families:
     GROUPED = ("grouped_gemm",)
     ELEMENTWISE = ("rmsnorm", "silu_mul", "rope_append", "embedding", "residual_add", "rmsnorm_exact", "latent_prep",
                    "head_cols", "scale_", "moe_route", "moe_sort", "moe_combine", "clamped_gate_mul", "cast_rows",
-                   "post_norm_add", "relu_squared", "scaled_sum_", "qk_norm_pack", "gated_part_norm")
-    RECURRENT = ("short_conv", "short_conv_carry", "ssd_scan")
+                   "post_norm_add", "relu_squared", "scaled_sum_", "qk_norm_pack", "gated_part_norm", "head_norm_gate",
+                   "streams_step", "head_norm_pack", "head_gate_cols")
+    RECURRENT = ("short_conv", "short_conv_carry", "ssd_scan", "delta_rule")
 
     def __init__(self):
         self.spans = []
@@ -422,6 +423,67 @@ def zabunex_work(s, n_layers, tokens, batch=0, kv_tokens=0, elt=2) -> dict:
             "recurrent": 2.0 * batch * n_par * 2 * state * 4 / elt}
 
 
+# Layers of the Vepitar design at the Zabunex sizes: to every four layers three of the
+# generalized delta rule and one of the sigmoid attention (convolutions of four taps, a window
+# as long as Zabunex's chunk), the residual stream in two copies, the first layer's feed-forward
+# dense and the others' a mixture of sixteen ungated experts of which a token uses four, as wide
+# together as Zabunex's feed-forward.  Beside it Zabunex layers of the same width, heads and
+# feed-forward: the closest design that the engine serves (an attention with convolutions
+# beside a recurrence with a float32 state per request).
+VEPITAR_SIZES = {
+    "2048-wide": dict(ZABUNEX_SIZES["2048-wide"], delta_heads=32, delta_dim=64, decay_rank=64, experts=16, top=4,
+                      expert_ff=2048, conv=4),
+    "4096-wide": dict(ZABUNEX_SIZES["4096-wide"], delta_heads=64, delta_dim=64, decay_rank=64, experts=16, top=4,
+                      expert_ff=4096, conv=4),
+}
+
+
+def vepitar_layer_kinds(n_layers):
+    return ["attention" if i % 4 == 1 else "general_delta" for i in range(n_layers)]
+
+
+def vepitar_config(s, n_layers, window):
+    delta = dict(heads=s["delta_heads"], dim=s["delta_dim"], decay_rank=s["decay_rank"])
+    attention = dict(heads=s["heads"], kv_heads=s["kv_heads"], dim=s["dim"], vdim=s["dim"], scale=s["dim"] ** -0.5,
+                     conv=s["conv"], mask=dict(size=window or s["chunk"]))
+    moe = dict(kind="moe", router=dict(experts=s["experts"], top=s["top"]), expert=dict(ff=s["expert_ff"]))
+    layers = [dict(type=kind, mixer=attention if kind == "attention" else delta,
+                   mlp=dict(kind="dense", ff=s["llama_ff"]) if i == 0 else moe)
+              for i, kind in enumerate(vepitar_layer_kinds(n_layers))]
+    return dict(architecture="Vepitar", vocab=COMPARISON_VOCAB, width=s["width"], norm=dict(eps=1e-6), streams=2,
+                residual_mult=0.5, max_positions=8192, layers=layers)
+
+
+def vepitar_work(s, n_layers, tokens, batch=0, kv_tokens=0, elt=2, window=0) -> dict:
+    """As ``zabunex_work``; the family ``recurrent`` is the convolutions and the delta rule
+    (nine float32 operations per token and entry of a head's state: the sum along the unit
+    key, the update and the read), whose decode step reads and writes every request's state."""
+    d, h, kv, D = s["width"], s["heads"], s["kv_heads"], s["dim"]
+    kinds = vepitar_layer_kinds(n_layers)
+    n_att, n_delta = kinds.count("attention"), kinds.count("general_delta")
+    n_dense, n_moe = 1, n_layers - 1
+    inner = s["delta_heads"] * s["delta_dim"]
+    att = d * ((h + 2 * kv) * D + h) + h * D * d
+    delta = d * (5 * inner + s["decay_rank"]) + inner * d
+    linear = n_att * att + n_delta * delta + n_dense * 3 * d * s["llama_ff"] + n_moe * d * s["experts"]
+    expert = 2 * d * s["expert_ff"]
+    state = s["delta_heads"] * s["delta_dim"] * s["delta_dim"]
+    span = window or s["chunk"]
+    if batch == 0:
+        seen = min(tokens, span)
+        return {"gemm": 2.0 * tokens * linear + 2.0 * COMPARISON_VOCAB * d,
+                "grouped": 2.0 * tokens * n_moe * s["top"] * expert,
+                "attention": tokens * h * D * (4.0 * seen - 2.0 * seen * seen / tokens) * n_att,
+                "recurrent": tokens * (n_delta * (9.0 * state + 2.0 * inner * s["decay_rank"])
+                                       + n_att * 2.0 * s["conv"] * (h + 2 * kv) * D)}
+    per_request = kv_tokens / batch
+    used = min(s["experts"], batch * s["top"])
+    return {"gemm": 2.0 * (linear + COMPARISON_VOCAB * d),
+            "grouped": 2.0 * n_moe * used * expert,
+            "attention": 2.0 * 2 * kv * D * batch * min(per_request, span) * n_att,
+            "recurrent": 2.0 * batch * n_delta * 2 * state * 4 / elt}
+
+
 DESIGNS = {
     "kavuvik": dict(label="Kavuvik", sizes=lambda: KAVUVIK_SIZES, config=lambda s, n, w: kavuvik_config(s, n, w),
                     llama=lambda s, n: closest_llama_config(s, n),
@@ -429,6 +491,10 @@ DESIGNS = {
     "zabunex": dict(label="Zabunex", sizes=lambda: ZABUNEX_SIZES, config=lambda s, n, w: zabunex_config(s, n, w),
                     llama=lambda s, n: llama_beside_zabunex(s, n),
                     work=lambda s, n, t, b, kv, elt: zabunex_work(s, n, t, b, kv, elt)),
+    "vepitar": dict(label="Vepitar", sizes=lambda: VEPITAR_SIZES, config=lambda s, n, w: vepitar_config(s, n, w),
+                    beside=dict(key="zabunex", label="Zabunex", config=lambda s, n: zabunex_config(s, n, 0),
+                                work=lambda s, n, t, b, kv, elt: zabunex_work(s, n, t, b, kv, elt)),
+                    work=lambda s, n, t, b, kv, elt, w=0: vepitar_work(s, n, t, b, kv, elt, w)),
 }
 
 
@@ -534,21 +600,32 @@ def design_comparison(args) -> dict:
         if args.sizes and name not in args.sizes.split(","):
             continue
         _, new = parse_config(design["config"](s, n_layers, args.window))
-        llama = LlamaConfig(**design["llama"](s, n_layers))
         print(f"[bench] {name}: {label}", file=sys.stderr, flush=True)
-        k = measure(new, lambda t, b=0, kv=0, elt=2, s=s: design["work"](s, n_layers, t, b, kv, elt))
-        print(f"[bench] {name}: Llama", file=sys.stderr, flush=True)
-        l = None if args.only_new else measure(llama, lambda t, b=0, kv=0, elt=2, c=llama: llama_work(c, n_layers, t, b, kv))
-        sizes[name] = {"shape": s, args.workload: k, "llama": l}
+        if args.workload == "vepitar":
+            k = measure(new, lambda t, b=0, kv=0, elt=2, s=s: design["work"](s, n_layers, t, b, kv, elt, args.window))
+        else:
+            k = measure(new, lambda t, b=0, kv=0, elt=2, s=s: design["work"](s, n_layers, t, b, kv, elt))
+        other = design.get("beside")
+        print(f"[bench] {name}: {other['label'] if other else 'Llama'}", file=sys.stderr, flush=True)
+        if args.only_new:
+            l = None
+        elif other:
+            _, cfg_other = parse_config(other["config"](s, n_layers))
+            l = measure(cfg_other, lambda t, b=0, kv=0, elt=2, s=s: other["work"](s, n_layers, t, b, kv, elt))
+        else:
+            llama = LlamaConfig(**design["llama"](s, n_layers))
+            l = measure(llama, lambda t, b=0, kv=0, elt=2, c=llama: llama_work(c, n_layers, t, b, kv))
+        sizes[name] = {"shape": s, args.workload: k, (other["key"] if other else "llama"): l}
     first_name = next(iter(sizes))
     first = sizes[first_name][args.workload]["decode"]["batch8"]
+    beside_label = design["beside"]["label"] if design.get("beside") else "Llama"
     return {
-        "metric": f"decode tokens per second of {label} layers ({first_name}, batch 8), beside Llama layers of equal size",
+        "metric": f"decode tokens per second of {label} layers ({first_name}, batch 8), beside {beside_label} layers of equal size",
         "value": first["tok_per_s"], "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": first["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
         "data": "synthetic: seeded uniform-random token ids, random weights N(0, 0.02)",
-        "config": {"model": f"{label} and Llama layers", "layers": n_layers, "global_batch": 8, "seq_len": context,
+        "config": {"model": f"{label} and {beside_label} layers", "layers": n_layers, "global_batch": 8, "seq_len": context,
                    "prefill_tokens": prompt, "window": args.window, "vocab_size": COMPARISON_VOCAB,
                    "hip_graph": not args.no_graph, "parallelism": "single GPU"},
         "sizes": sizes,
@@ -577,9 +654,10 @@ def main() -> int:
                          "by default (scheduling_steps_ahead); 0: read every step's tokens before the next is put together")
     ap.add_argument("--sampling", default="greedy", choices=["greedy", "temperature", "top_p", "top_k", "all"],
                     help="how the decode steps sample (the contract's line is greedy)")
-    ap.add_argument("--workload", default="decode8b", choices=["decode8b", "mixed3b", "llama70b", "kavuvik", "zabunex"],
+    ap.add_argument("--workload", default="decode8b", choices=["decode8b", "mixed3b", "llama70b", "kavuvik", "zabunex", "vepitar"],
                     help="decode8b: the headline line; mixed3b and llama70b run requests through the scheduler; "
-                         "kavuvik, zabunex: prefill and decode of that design's layers at two sizes beside the closest Llama layers")
+                         "kavuvik, zabunex: prefill and decode of that design's layers at two sizes beside the closest Llama layers; "
+                         "vepitar: the same beside Zabunex layers of equal size")
     ap.add_argument("--sizes", default="", help="kavuvik: only these sizes (names with commas between them)")
     ap.add_argument("--only-new", action="store_true", help="kavuvik: leave the Llama layers out (for profiles)")
     ap.add_argument("--window", type=int, default=0,

@@ -108,10 +108,16 @@ def gated_feed_forward(h, w, pre):
     return (z * torch.sigmoid(z) * (h @ w[pre + "up"].T)) @ w[pre + "down"].T
 
 
-def routed_experts(h, w, pre, mlp):
-    """Softmax over all experts, the ``top`` largest, their scores over their sum."""
+def routed_experts(h, w, pre, mlp, margins_out=None):
+    """Softmax over all experts, the ``top`` largest, their scores over their sum.
+    ``margins_out`` receives, per token, how far the last chosen expert's logit lies above
+    the first that is not chosen."""
     E, top = mlp["router"]["experts"], mlp["router"]["top"]
-    scores = torch.softmax(h @ w[pre + "router"].T, -1)
+    logits = h @ w[pre + "router"].T
+    if margins_out is not None and top < E:
+        ranked = logits.sort(-1, descending=True).values
+        margins_out.append(ranked[:, top - 1] - ranked[:, top])
+    scores = torch.softmax(logits, -1)
     chosen_s, chosen = torch.topk(scores, top, dim=-1)
     weights = chosen_s / (chosen_s.sum(-1, keepdim=True) + 1e-20)
     out = torch.zeros_like(h)
@@ -123,10 +129,10 @@ def routed_experts(h, w, pre, mlp):
     return out
 
 
-def feed_forward(h, w, pre, mlp):
+def feed_forward(h, w, pre, mlp, margins_out=None):
     if mlp["kind"] == "dense":
         return gated_feed_forward(h, w, pre)
-    return routed_experts(h, w, pre, mlp)
+    return routed_experts(h, w, pre, mlp, margins_out)
 
 
 def connection_read(streams, w_in):
@@ -141,9 +147,13 @@ def connection_write(streams, y, w_mix, w_out, mult):
     return [sum(w_mix[s, t] * streams[s] for s in range(n)) + mult * w_out[t] * y for t in range(n)]
 
 
-def forward(cfg: dict, w: dict, tokens, dtype=torch.float64, layers_out: list | None = None):
+def forward(cfg: dict, w: dict, tokens, dtype=torch.float64, layers_out: list | None = None, round_inputs=None,
+            margins_out: list | None = None):
     """Logits ``[T, vocab]`` of one request's tokens.  ``layers_out`` receives the stream
-    after every layer (the sum of the copies where there are several)."""
+    after every layer (the sum of the copies where there are several).  ``round_inputs``: an
+    element type that every part's normed input is rounded to on the way (how far the logits
+    move then says how sensitive a position is to arithmetic in that type).  ``margins_out``
+    receives every routed feed-forward's margins (see ``routed_experts``)."""
     w = {n: (t.to(dtype) if t.is_floating_point() else t) for n, t in w.items()}
     eps = cfg["norm"]["eps"]
     m = cfg.get("residual_mult", 1.0)
@@ -161,8 +171,10 @@ def forward(cfg: dict, w: dict, tokens, dtype=torch.float64, layers_out: list | 
             else:
                 inp = x
             h = norm_around_zero(inp, w[f"{pre}norm{q}"], eps)
+            if round_inputs is not None:
+                h = h.to(round_inputs).to(dtype)
             if q == 2:
-                y = feed_forward(h, w, pre + "mlp.", layer["mlp"])
+                y = feed_forward(h, w, pre + "mlp.", layer["mlp"], margins_out)
             elif layer["type"] == "attention":
                 y = sigmoid_window_attention(h, w, pre + "mix.", layer["mixer"], eps)
             elif layer["type"] == "general_delta":
@@ -178,6 +190,26 @@ def forward(cfg: dict, w: dict, tokens, dtype=torch.float64, layers_out: list | 
     if streams is not None:
         x = sum(streams)
     return norm_around_zero(x, w["final.norm"], eps) @ w["embed"].T
+
+
+def tokens_with_clear_routing(cfg, w, tokens, margin=0.1, seed=0, tries=400):
+    """``tokens`` with as few replaced as it takes for no router of the model to choose between
+    two experts whose logits lie closer than ``margin``: arithmetic in 16 bits moves a logit by
+    a few hundredths, and a choice that turns over makes another model of it.  The first
+    token with such a call is drawn anew until there is none (earlier tokens stay as they are:
+    the model is causal)."""
+    gen = torch.Generator().manual_seed(seed)
+    ids = list(tokens)
+    for _ in range(tries):
+        margins = []
+        forward(cfg, w, ids, margins_out=margins)
+        if not margins:
+            return ids
+        close = (torch.stack(margins).min(0).values < margin).nonzero()
+        if close.numel() == 0:
+            return ids
+        ids[int(close[0])] = int(torch.randint(0, cfg["vocab"], (1,), generator=gen))
+    raise RuntimeError("no sequence without a close call of a router")
 
 
 # ---- configurations, tensors and folders for the tests ------------------------------------------
