@@ -8,8 +8,9 @@
 // where both middle terms read the old state.  The state lives in float32 rows, one per
 // request slot, and a step's tokens come as a flat batch of segments, as for the other
 // recurrences.  Three kernels: what a token contributes (decay, erase vector, unit key; all
-// tokens side by side), the walk over the tokens of every segment, and the norm and gate of
-// the walk's result.  Everything here is float32 whatever the activations' type is.
+// tokens side by side), the walk over the tokens of every segment (or, where every segment
+// is one token, a kernel that reads and writes each state once in whole rows), and the norm
+// and gate of the walk's result.  Everything here is float32 whatever the activations' type is.
 #include "hal_common.h"
 #include "hal_api.h"
 
@@ -18,51 +19,101 @@
 
 __device__ __forceinline__ float delta_sigmoid(float x) { return 1.0f / (1.0f + expf(-x)); }
 
-// ---- a workgroup a (token, head); thread c a key channel.  pre [T][H][5][DP], zero beyond D.
+// ---- a workgroup takes DELTA_PREP_TOKENS tokens of one head; thread c a key channel, whose
+// row of W2 it holds in registers (DELTA_PREP_RANK entries at a time) for all the tokens.
+// pre [T][H][5][DP], zero beyond D.
+#define DELTA_PREP_TOKENS 16
+#define DELTA_PREP_RANK 32
 __global__ void delta_prep_kernel(const float* __restrict__ r, int ldr, const float* __restrict__ k, int ldk,
                                   const float* __restrict__ a_raw, int lda, const float* __restrict__ x1, int ldx1,
                                   const void* __restrict__ w2, const void* __restrict__ w0,
                                   const void* __restrict__ a_bias, int w_dtype, int lora, float decay_rate,
-                                  float unit_eps, float* __restrict__ pre, int H, int D, int DP) {
+                                  float unit_eps, float* __restrict__ pre, int n_tokens, int H, int D, int DP) {
   __shared__ float scratch[16];
-  __shared__ float tl[DELTA_MAX_LORA];
-  const size_t t = blockIdx.x;
+  __shared__ float tl[DELTA_PREP_TOKENS][DELTA_PREP_RANK];
+  const int t0 = blockIdx.x * DELTA_PREP_TOKENS;
+  const int nt = n_tokens - t0 < DELTA_PREP_TOKENS ? n_tokens - t0 : DELTA_PREP_TOKENS;
   const int h = blockIdx.y, c = threadIdx.x;
-  for (int j = threadIdx.x; j < lora; j += blockDim.x) tl[j] = tanhf(x1[t * ldx1 + j]);
   const bool live = c < D;
-  const size_t ch = (size_t)h * D + c;
-  const float kc = live ? k[t * ldk + ch] : 0.f;
-  const float kk = block_sum(kc * kc, scratch);  // (its barrier also covers tl)
-  if (c >= DP) return;
-  float* dst = pre + ((t * H + h) * DELTA_VECTORS) * DP + c;
-  float decay = 0.f, au = 0.f, u = 0.f, rc = 0.f;
-  if (live) {
-    float z = load_as_f32(w0, w_dtype, ch);
-    for (int j = 0; j < lora; ++j) z = fmaf(load_as_f32(w2, w_dtype, ch * lora + j), tl[j], z);
-    decay = expf(-decay_rate * delta_sigmoid(z));
-    u = kc / sqrtf(kk + unit_eps);
-    au = delta_sigmoid(a_raw[t * lda + ch] + load_as_f32(a_bias, w_dtype, ch)) * u;
-    rc = r[t * ldr + ch];
+  const size_t ch = (size_t)h * D + (live ? c : 0);
+  float z[DELTA_PREP_TOKENS];
+  const float z0 = load_as_f32(w0, w_dtype, ch);
+#pragma unroll
+  for (int i = 0; i < DELTA_PREP_TOKENS; ++i) z[i] = z0;
+  for (int j0 = 0; j0 < lora; j0 += DELTA_PREP_RANK) {
+    const int nj = lora - j0 < DELTA_PREP_RANK ? lora - j0 : DELTA_PREP_RANK;
+    __syncthreads();
+    for (int i = threadIdx.x; i < DELTA_PREP_TOKENS * DELTA_PREP_RANK; i += blockDim.x) {
+      const int tok = i / DELTA_PREP_RANK, j = i % DELTA_PREP_RANK;
+      tl[tok][j] = (tok < nt && j < nj) ? tanhf(x1[(size_t)(t0 + tok) * ldx1 + j0 + j]) : 0.f;
+    }
+    float w[DELTA_PREP_RANK];
+#pragma unroll
+    for (int j = 0; j < DELTA_PREP_RANK; ++j) w[j] = j < nj ? load_as_f32(w2, w_dtype, ch * lora + j0 + j) : 0.f;
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < DELTA_PREP_TOKENS; ++i) {
+#pragma unroll
+      for (int j = 0; j < DELTA_PREP_RANK; j += 4) {
+        const float4 x4 = *(const float4*)&tl[i][j];
+        z[i] = fmaf(w[j], x4.x, z[i]);
+        z[i] = fmaf(w[j + 1], x4.y, z[i]);
+        z[i] = fmaf(w[j + 2], x4.z, z[i]);
+        z[i] = fmaf(w[j + 3], x4.w, z[i]);
+      }
+    }
   }
-  dst[0] = decay;
-  dst[DP] = au;
-  dst[2 * DP] = u;
-  dst[3 * DP] = kc;
-  dst[4 * DP] = rc;
+  const float ab = load_as_f32(a_bias, w_dtype, ch);
+#pragma unroll
+  for (int i = 0; i < DELTA_PREP_TOKENS; ++i) {
+    if (i >= nt) break;  // (the same for every thread of the workgroup)
+    const size_t t = t0 + i;
+    const float kc = live ? k[t * ldk + ch] : 0.f;
+    const float kk = block_sum(kc * kc, scratch);
+    if (c >= DP) continue;
+    float* dst = pre + ((t * H + h) * DELTA_VECTORS) * DP + c;
+    float decay = 0.f, au = 0.f, u = 0.f, rc = 0.f;
+    if (live) {
+      decay = expf(-decay_rate * delta_sigmoid(z[i]));
+      u = kc / sqrtf(kk + unit_eps);
+      au = delta_sigmoid(a_raw[t * lda + ch] + ab) * u;
+      rc = r[t * ldr + ch];
+    }
+    dst[0] = decay;
+    dst[DP] = au;
+    dst[2 * DP] = u;
+    dst[3 * DP] = kc;
+    dst[4 * DP] = rc;
+  }
+}
+
+// The sum of a value over the wave's four quarters of 16 lanes, in every lane: two swaps of
+// lane halves inside the vector unit (rows 1 and 3 against rows 0 and 2, then the upper 32
+// lanes against the lower), each followed by an addition.
+__device__ __forceinline__ float quarters_sum(float x) {
+  const unsigned b = __float_as_uint(x);
+  const auto p = __builtin_amdgcn_permlane16_swap(b, b, false, false);
+  const unsigned s = __float_as_uint(__uint_as_float(p[0]) + __uint_as_float(p[1]));
+  const auto q = __builtin_amdgcn_permlane32_swap(s, s, false, false);
+  return __uint_as_float(q[0]) + __uint_as_float(q[1]);
 }
 
 // ---- the walk: a wave takes 16 value channels of one head of one segment; the key channels
 // are split over the wave's four quarters, so a lane holds NREG numbers of its channel's
 // column of the state, and the two sums over the key channels (u^T S and S^T r) cross the
-// quarters with two exchanges each.  A token's five vectors (shared by the lanes) go through
-// LDS, the next token's on their way meanwhile.
+// quarters with two swaps of lane halves each.  The tokens' five vectors (shared by the lanes) go through
+// LDS in blocks of TB tokens, the next block's on their way from memory while one is walked,
+// so that the memory's latency is paid once a block and not once a token.
 template <int NREG>
 __global__ void __launch_bounds__(HAL_WAVE)
 delta_scan_kernel(const float* __restrict__ pre, const float* __restrict__ v, int ldv, float* __restrict__ state,
                   const int* __restrict__ seg_q_start, const int* __restrict__ seg_q_len,
                   const int* __restrict__ token_slot, float* __restrict__ o, int H, int D) {
-  constexpr int DP = NREG * 4, TOTAL = DELTA_VECTORS * DP, PER = (TOTAL + HAL_WAVE - 1) / HAL_WAVE;
-  __shared__ __align__(16) float vec[2][TOTAL];
+  constexpr int DP = NREG * 4, TOTAL = DELTA_VECTORS * DP;
+  constexpr int TB = DP <= 64 ? 8 : DP == 128 ? 4 : 2;
+  constexpr int PER = TB * TOTAL / HAL_WAVE;
+  static_assert(TB * TOTAL % HAL_WAVE == 0, "a block of tokens is whole loads of the wave");
+  __shared__ __align__(16) float vec[2][TB * TOTAL];
   const int s = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int col = blockIdx.z * 16 + lane % 16, row0 = (lane / 16) * NREG;
   const int t0 = seg_q_start[s], n = seg_q_len[s];
@@ -73,68 +124,63 @@ delta_scan_kernel(const float* __restrict__ pre, const float* __restrict__ v, in
 #pragma unroll
   for (int i = 0; i < NREG; ++i) S[i] = (live && row0 + i < D) ? st[(size_t)(row0 + i) * D] : 0.f;
 
-  float next[PER];
-  auto ask = [&](int t) {
-    const float* src = pre + ((size_t)t * H + h) * TOTAL;
+  float next[PER], v_next[TB];
+  auto ask = [&](int t, int cnt) {  // tokens t .. t + cnt - 1
 #pragma unroll
     for (int u = 0; u < PER; ++u) {
-      const int i = lane + u * HAL_WAVE;
-      next[u] = i < TOTAL ? src[i] : 0.f;
+      const int i = lane + u * HAL_WAVE, tok = i / TOTAL;
+      next[u] = tok < cnt ? pre[((size_t)(t + tok) * H + h) * TOTAL + (i - tok * TOTAL)] : 0.f;
     }
-  };
-  auto put = [&](int buf) {
 #pragma unroll
-    for (int u = 0; u < PER; ++u) {
-      const int i = lane + u * HAL_WAVE;
-      if (i < TOTAL) vec[buf][i] = next[u];
-    }
+    for (int j = 0; j < TB; ++j) v_next[j] = (live && j < cnt) ? v[(size_t)(t + j) * ldv + (size_t)h * D + col] : 0.f;
   };
-  ask(t0);
-  float v_next = live ? v[(size_t)t0 * ldv + (size_t)h * D + col] : 0.f;
-  for (int i = 0; i < n; ++i) {
-    const int t = t0 + i, buf = i & 1;
-    put(buf);
-    const float vv = v_next;
-    if (i + 1 < n) {
-      ask(t + 1);
-      v_next = live ? v[(size_t)(t + 1) * ldv + (size_t)h * D + col] : 0.f;
-    }
+  ask(t0, n < TB ? n : TB);
+  for (int b = 0; b * TB < n; ++b) {
+    const int base = t0 + b * TB, left = n - b * TB, cnt = left < TB ? left : TB;
+    float* blk = vec[b & 1];
+#pragma unroll
+    for (int u = 0; u < PER; ++u) blk[lane + u * HAL_WAVE] = next[u];
+    float vv[TB];
+#pragma unroll
+    for (int j = 0; j < TB; ++j) vv[j] = v_next[j];
+    if (left > TB) ask(base + TB, left - TB < TB ? left - TB : TB);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    const float* wv = vec[buf] + row0;
-    float d0 = 0.f, d1 = 0.f;
 #pragma unroll
-    for (int j = 0; j < NREG; j += 4) {
-      const float4 u4 = *(const float4*)(wv + 2 * DP + j);
-      d0 = fmaf(S[j], u4.x, d0);
-      d1 = fmaf(S[j + 1], u4.y, d1);
-      d0 = fmaf(S[j + 2], u4.z, d0);
-      d1 = fmaf(S[j + 3], u4.w, d1);
-    }
-    float dot = d0 + d1;  // u^T S_(t-1) of this column, a quarter of it
-    dot += __shfl_xor(dot, 16, HAL_WAVE);
-    dot += __shfl_xor(dot, 32, HAL_WAVE);
-    float a0 = 0.f, a1 = 0.f;
+    for (int jt = 0; jt < TB; ++jt) {
+      if (jt >= cnt) break;
+      const float* wv = blk + jt * TOTAL + row0;
+      float d0 = 0.f, d1 = 0.f;
 #pragma unroll
-    for (int j = 0; j < NREG; j += 4) {
-      const float4 w4 = *(const float4*)(wv + j);
-      const float4 e4 = *(const float4*)(wv + DP + j);
-      const float4 k4 = *(const float4*)(wv + 3 * DP + j);
-      const float4 r4 = *(const float4*)(wv + 4 * DP + j);
-      S[j] = fmaf(w4.x, S[j], fmaf(-e4.x, dot, k4.x * vv));
-      a0 = fmaf(S[j], r4.x, a0);
-      S[j + 1] = fmaf(w4.y, S[j + 1], fmaf(-e4.y, dot, k4.y * vv));
-      a1 = fmaf(S[j + 1], r4.y, a1);
-      S[j + 2] = fmaf(w4.z, S[j + 2], fmaf(-e4.z, dot, k4.z * vv));
-      a0 = fmaf(S[j + 2], r4.z, a0);
-      S[j + 3] = fmaf(w4.w, S[j + 3], fmaf(-e4.w, dot, k4.w * vv));
-      a1 = fmaf(S[j + 3], r4.w, a1);
+      for (int j = 0; j < NREG; j += 4) {
+        const float4 u4 = *(const float4*)(wv + 2 * DP + j);
+        d0 = fmaf(S[j], u4.x, d0);
+        d1 = fmaf(S[j + 1], u4.y, d1);
+        d0 = fmaf(S[j + 2], u4.z, d0);
+        d1 = fmaf(S[j + 3], u4.w, d1);
+      }
+      const float dot = quarters_sum(d0 + d1);  // u^T S_(t-1) of this column
+      const float val = vv[jt];
+      float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+      for (int j = 0; j < NREG; j += 4) {
+        const float4 w4 = *(const float4*)(wv + j);
+        const float4 e4 = *(const float4*)(wv + DP + j);
+        const float4 k4 = *(const float4*)(wv + 3 * DP + j);
+        const float4 r4 = *(const float4*)(wv + 4 * DP + j);
+        S[j] = fmaf(w4.x, S[j], fmaf(-e4.x, dot, k4.x * val));
+        a0 = fmaf(S[j], r4.x, a0);
+        S[j + 1] = fmaf(w4.y, S[j + 1], fmaf(-e4.y, dot, k4.y * val));
+        a1 = fmaf(S[j + 1], r4.y, a1);
+        S[j + 2] = fmaf(w4.z, S[j + 2], fmaf(-e4.z, dot, k4.z * val));
+        a0 = fmaf(S[j + 2], r4.z, a0);
+        S[j + 3] = fmaf(w4.w, S[j + 3], fmaf(-e4.w, dot, k4.w * val));
+        a1 = fmaf(S[j + 3], r4.w, a1);
+      }
+      const float acc = quarters_sum(a0 + a1);
+      if (live && lane < 16) o[(size_t)(base + jt) * H * D + (size_t)h * D + col] = acc;
     }
-    float acc = a0 + a1;
-    acc += __shfl_xor(acc, 16, HAL_WAVE);
-    acc += __shfl_xor(acc, 32, HAL_WAVE);
-    if (live && lane < 16) o[(size_t)t * H * D + (size_t)h * D + col] = acc;
   }
   if (live) {
 #pragma unroll
@@ -143,10 +189,75 @@ delta_scan_kernel(const float* __restrict__ pre, const float* __restrict__ v, in
   }
 }
 
+// ---- a step in which every request brings one token: a workgroup of 256 threads takes one
+// head of one request, reads and writes its state once in rows of 16 bytes a thread (a wave
+// covers whole rows), and the two sums over the key channels cross the waves through LDS.
+// D is 32, 64 or 128; a thread holds R rows of four neighbouring value channels.
+template <int D>
+__global__ void __launch_bounds__(256)
+delta_step_kernel(const float* __restrict__ pre, const float* __restrict__ v, int ldv, float* __restrict__ state,
+                  const int* __restrict__ token_slot, float* __restrict__ o, int H) {
+  constexpr int CG = D / 4, RG = 256 / CG, R = D / RG, TOTAL = DELTA_VECTORS * D, WAVES = 256 / HAL_WAVE;
+  static_assert(CG <= HAL_WAVE && 256 % CG == 0 && D % RG == 0, "a head of 32, 64 or 128 channels");
+  __shared__ __align__(16) float vec[TOTAL];
+  __shared__ float4 red[2][WAVES][CG];
+  const int t = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+  const int cg = tid % CG, rg = tid / CG, col = cg * 4, wave = tid / HAL_WAVE;
+  const float* src = pre + ((size_t)t * H + h) * TOTAL;
+  for (int i = tid; i < TOTAL; i += 256) vec[i] = src[i];
+  float* st = state + ((size_t)token_slot[t] * H + h) * D * D + col;
+  float4 S[R];
+#pragma unroll
+  for (int j = 0; j < R; ++j) S[j] = *(const float4*)(st + (size_t)(rg + j * RG) * D);
+  const float* vr = v + (size_t)t * ldv + (size_t)h * D + col;
+  const float4 vv = make_float4(vr[0], vr[1], vr[2], vr[3]);
+  __syncthreads();
+  auto across = [&](float4 x, int which) {  // the sum over all row groups, in every thread
+#pragma unroll
+    for (int m = CG; m < HAL_WAVE; m <<= 1) {
+      x.x += __shfl_xor(x.x, m, HAL_WAVE);
+      x.y += __shfl_xor(x.y, m, HAL_WAVE);
+      x.z += __shfl_xor(x.z, m, HAL_WAVE);
+      x.w += __shfl_xor(x.w, m, HAL_WAVE);
+    }
+    if (tid % HAL_WAVE < CG) red[which][wave][cg] = x;
+    __syncthreads();
+    float4 sum = red[which][0][cg];
+#pragma unroll
+    for (int w = 1; w < WAVES; ++w) {
+      const float4 y = red[which][w][cg];
+      sum.x += y.x, sum.y += y.y, sum.z += y.z, sum.w += y.w;
+    }
+    return sum;
+  };
+  float4 d = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+  for (int j = 0; j < R; ++j) {
+    const float u = vec[2 * D + rg + j * RG];
+    d.x = fmaf(S[j].x, u, d.x), d.y = fmaf(S[j].y, u, d.y), d.z = fmaf(S[j].z, u, d.z), d.w = fmaf(S[j].w, u, d.w);
+  }
+  const float4 dot = across(d, 0);
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+  for (int j = 0; j < R; ++j) {
+    const int row = rg + j * RG;
+    const float w = vec[row], e = vec[D + row], k = vec[3 * D + row], r = vec[4 * D + row];
+    S[j].x = fmaf(w, S[j].x, fmaf(-e, dot.x, k * vv.x));
+    S[j].y = fmaf(w, S[j].y, fmaf(-e, dot.y, k * vv.y));
+    S[j].z = fmaf(w, S[j].z, fmaf(-e, dot.z, k * vv.z));
+    S[j].w = fmaf(w, S[j].w, fmaf(-e, dot.w, k * vv.w));
+    acc.x = fmaf(S[j].x, r, acc.x), acc.y = fmaf(S[j].y, r, acc.y), acc.z = fmaf(S[j].z, r, acc.z), acc.w = fmaf(S[j].w, r, acc.w);
+    *(float4*)(st + (size_t)row * D) = S[j];
+  }
+  const float4 out = across(acc, 1);
+  if (tid < CG) *(float4*)(o + (size_t)t * H * D + (size_t)h * D + col) = out;
+}
+
 // r, k, v, a_raw: float32 [T, H * D] (row-strided views allowed), x1 float32 [T, lora];
 // w2 [H * D, lora], w0 and a_bias [H * D] of one element type; state float32
 // [slots][H][D][D], read and left as the step's last state; pre: room for T * H * 5 * DP
-// floats with DP = D rounded up to 16, 32, 64, 128 or 256; o float32 [T, H * D].
+// floats with DP = D rounded up to 16, 32, 64, 128 or 256; o float32 [T, H * D].  No segment
+// is empty: a step with as many tokens as segments brings one token a segment.
 extern "C" int hal_delta_rule(const float* r, int ldr, const float* k, int ldk, const float* v, int ldv,
                               const float* a_raw, int lda, const float* x1, int ldx1, const void* w2,
                               const void* w0, const void* a_bias, int w_dtype, int lora, float decay_rate,
@@ -163,8 +274,20 @@ extern "C" int hal_delta_rule(const float* r, int ldr, const float* k, int ldk, 
   HAL_REQUIRE(w_dtype == HAL_F32 || w_dtype == HAL_BF16, "hal_delta_rule: dtype %d", w_dtype);
   if (n_tokens == 0 || n_segs == 0) return 0;
   const int DP = D <= 16 ? 16 : D <= 32 ? 32 : D <= 64 ? 64 : D <= 128 ? 128 : 256;
-  hipLaunchKernelGGL(delta_prep_kernel, dim3(n_tokens, H), dim3(DP < 64 ? 64 : DP), 0, stream, r, ldr, k, ldk, a_raw,
-                     lda, x1, ldx1, w2, w0, a_bias, w_dtype, lora, decay_rate, unit_eps, pre, H, D, DP);
+  hipLaunchKernelGGL(delta_prep_kernel, dim3((n_tokens + DELTA_PREP_TOKENS - 1) / DELTA_PREP_TOKENS, H),
+                     dim3(DP < 64 ? 64 : DP), 0, stream, r, ldr, k, ldk, a_raw, lda, x1, ldx1, w2, w0, a_bias, w_dtype,
+                     lora, decay_rate, unit_eps, pre, n_tokens, H, D, DP);
+  if (n_tokens == n_segs && (D == 32 || D == 64 || D == 128)) {  // (DP == D for these)
+    const dim3 heads(n_tokens, H);
+    if (D == 32)
+      hipLaunchKernelGGL(delta_step_kernel<32>, heads, dim3(256), 0, stream, pre, v, ldv, state, token_slot, o, H);
+    else if (D == 64)
+      hipLaunchKernelGGL(delta_step_kernel<64>, heads, dim3(256), 0, stream, pre, v, ldv, state, token_slot, o, H);
+    else
+      hipLaunchKernelGGL(delta_step_kernel<128>, heads, dim3(256), 0, stream, pre, v, ldv, state, token_slot, o, H);
+    HAL_LAUNCH_CHECK();
+    return 0;
+  }
   const dim3 grid(n_segs, H, (D + 15) / 16);
 #define DELTA_SCAN(N_)                                                                                       \
   hipLaunchKernelGGL(delta_scan_kernel<N_>, grid, dim3(HAL_WAVE), 0, stream, pre, v, ldv, state, seg_q_start, \

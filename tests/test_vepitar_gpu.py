@@ -106,15 +106,18 @@ def step_arrays(gpu, cuts, slots):
 
 
 @pytest.mark.parametrize("stored", ["float32", "bfloat16"])
-@pytest.mark.parametrize("shape", [(4, 16, 8), (1, 48, 3), (5, 8, 6), (2, 24, 5), (2, 64, 4), (3, 80, 2), (1, 132, 7)])
+@pytest.mark.parametrize("shape", [(4, 16, 8), (1, 48, 3), (5, 8, 6), (2, 24, 5), (2, 64, 4), (3, 80, 2), (1, 132, 7),
+                                   (3, 32, 4), (2, 128, 3)])
 def test_delta_rule_in_steps(gpu, stored, shape):
     """The recurrence over two requests cut into steps of unequal sizes (single tokens, two,
-    many), in slots that are not in order, against the whole sequences; the state is carried
-    in float32 rows, and the rows of other slots hold NaN.  Heads of 8 to 132 channels: fewer
-    than a wave's quarter holds, and more than one block of value channels."""
+    many, more than a block of the walk), in slots that are not in order, against the whole
+    sequences; the state is carried in float32 rows, and the rows of other slots hold NaN.
+    Heads of 8 to 132 channels: fewer than a wave's quarter holds, and more than one block of
+    value channels; steps of single tokens alone take a kernel of their own for heads of 32,
+    64 and 128."""
     H, D, rank = shape
     n = H * D
-    T = {2: 45, 0: 21}
+    T = {2: 47, 0: 23}
     w2, w0, ab = (rand(n, rank, seed=1, scale=0.8).to(DT[stored]), rand(n, seed=2, scale=1.5).to(DT[stored]),
                   rand(n, seed=3).to(DT[stored]))
     rows = {s: rand(t, 3 + 4 * n + rank, seed=10 + s) for s, t in T.items()}
@@ -132,7 +135,7 @@ def test_delta_rule_in_steps(gpu, stored, shape):
     state = torch.full((4, H, D, D), float("nan"), device=gpu)
     state[0].zero_(), state[2].zero_()
     at = {2: 0, 0: 0}
-    for step in ({2: 1, 0: 2}, {2: 2}, {0: 1, 2: 1}, {0: 1, 2: 33}, {2: 8, 0: 17}):
+    for step in ({2: 1, 0: 2}, {2: 2}, {0: 1, 2: 1}, {0: 1, 2: 33}, {2: 1, 0: 1}, {2: 8, 0: 17}, {0: 1, 2: 1}):
         slots = list(step)
         cuts = [step[s] for s in slots]
         a = torch.cat([rows[s][at[s] : at[s] + step[s]] for s in slots]).to(gpu)[:, 3:]  # rows that begin off 16 bytes
