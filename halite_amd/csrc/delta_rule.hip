@@ -22,8 +22,8 @@ __device__ __forceinline__ float delta_sigmoid(float x) { return 1.0f / (1.0f + 
 // ---- a workgroup takes DELTA_PREP_TOKENS tokens of one head; thread c a key channel, whose
 // row of W2 it holds in registers (DELTA_PREP_RANK entries at a time) for all the tokens.
 // pre [T][H][5][DP], zero beyond D.
-#define DELTA_PREP_TOKENS 16
 #define DELTA_PREP_RANK 32
+template <int DELTA_PREP_TOKENS>
 __global__ void delta_prep_kernel(const float* __restrict__ r, int ldr, const float* __restrict__ k, int ldk,
                                   const float* __restrict__ a_raw, int lda, const float* __restrict__ x1, int ldx1,
                                   const void* __restrict__ w2, const void* __restrict__ w0,
@@ -64,11 +64,20 @@ __global__ void delta_prep_kernel(const float* __restrict__ r, int ldr, const fl
     }
   }
   const float ab = load_as_f32(a_bias, w_dtype, ch);
+  float kc_[DELTA_PREP_TOKENS], ar_[DELTA_PREP_TOKENS], rc_[DELTA_PREP_TOKENS];
+#pragma unroll
+  for (int i = 0; i < DELTA_PREP_TOKENS; ++i) {  // all of a thread's loads on their way at once
+    const bool have = live && i < nt;
+    const size_t t = t0 + i;
+    kc_[i] = have ? k[t * ldk + ch] : 0.f;
+    ar_[i] = have ? a_raw[t * lda + ch] : 0.f;
+    rc_[i] = have ? r[t * ldr + ch] : 0.f;
+  }
 #pragma unroll
   for (int i = 0; i < DELTA_PREP_TOKENS; ++i) {
     if (i >= nt) break;  // (the same for every thread of the workgroup)
     const size_t t = t0 + i;
-    const float kc = live ? k[t * ldk + ch] : 0.f;
+    const float kc = kc_[i];
     const float kk = block_sum(kc * kc, scratch);
     if (c >= DP) continue;
     float* dst = pre + ((t * H + h) * DELTA_VECTORS) * DP + c;
@@ -76,8 +85,8 @@ __global__ void delta_prep_kernel(const float* __restrict__ r, int ldr, const fl
     if (live) {
       decay = expf(-decay_rate * delta_sigmoid(z[i]));
       u = kc / sqrtf(kk + unit_eps);
-      au = delta_sigmoid(a_raw[t * lda + ch] + ab) * u;
-      rc = r[t * ldr + ch];
+      au = delta_sigmoid(ar_[i] + ab) * u;
+      rc = rc_[i];
     }
     dst[0] = decay;
     dst[DP] = au;
@@ -98,24 +107,32 @@ __device__ __forceinline__ float quarters_sum(float x) {
   return __uint_as_float(q[0]) + __uint_as_float(q[1]);
 }
 
-// ---- the walk: a wave takes 16 value channels of one head of one segment; the key channels
-// are split over the wave's four quarters, so a lane holds NREG numbers of its channel's
-// column of the state, and the two sums over the key channels (u^T S and S^T r) cross the
-// quarters with two swaps of lane halves each.  The tokens' five vectors (shared by the lanes) go through
-// LDS in blocks of TB tokens, the next block's on their way from memory while one is walked,
-// so that the memory's latency is paid once a block and not once a token.
-template <int NREG>
+// ---- the walk: a wave takes COLS (16 or 8) value channels of one head of one segment; the
+// key channels are split over the wave's 64 / COLS groups of lanes, so a lane holds NREG
+// numbers of its channel's column of the state, and the two sums over the key channels
+// (u^T S and S^T r) cross the groups inside the vector unit.  The tokens' five vectors
+// (shared by the lanes) go through LDS in blocks of TB tokens, the next block's on their way
+// from memory while one is walked, so that the memory's latency is paid once a block and not
+// once a token; a whole block is walked without a branch between its tokens.
+template <int COLS>
+__device__ __forceinline__ float groups_sum(float x) {
+  if (COLS == 8)  // lanes i and i ^ 8: a rotation by 8 inside every row of 16 lanes
+    x += __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(x), 0x128, 0xf, 0xf, false));
+  return quarters_sum(x);
+}
+
+template <int NREG, int COLS>
 __global__ void __launch_bounds__(HAL_WAVE)
 delta_scan_kernel(const float* __restrict__ pre, const float* __restrict__ v, int ldv, float* __restrict__ state,
                   const int* __restrict__ seg_q_start, const int* __restrict__ seg_q_len,
                   const int* __restrict__ token_slot, float* __restrict__ o, int H, int D) {
-  constexpr int DP = NREG * 4, TOTAL = DELTA_VECTORS * DP;
+  constexpr int DP = NREG * (HAL_WAVE / COLS), TOTAL = DELTA_VECTORS * DP;
   constexpr int TB = DP <= 64 ? 8 : DP == 128 ? 4 : 2;
   constexpr int PER = TB * TOTAL / HAL_WAVE;
-  static_assert(TB * TOTAL % HAL_WAVE == 0, "a block of tokens is whole loads of the wave");
-  __shared__ __align__(16) float vec[2][TB * TOTAL];
+  static_assert(TB * TOTAL % HAL_WAVE == 0 && NREG % 4 == 0, "a block of tokens is whole loads of the wave");
+  __shared__ __align__(16) float vec[2 * TB * TOTAL];
   const int s = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-  const int col = blockIdx.z * 16 + lane % 16, row0 = (lane / 16) * NREG;
+  const int col = blockIdx.z * COLS + lane % COLS, row0 = (lane / COLS) * NREG;
   const int t0 = seg_q_start[s], n = seg_q_len[s];
   if (n <= 0) return;
   const bool live = col < D;
@@ -134,12 +151,43 @@ delta_scan_kernel(const float* __restrict__ pre, const float* __restrict__ v, in
 #pragma unroll
     for (int j = 0; j < TB; ++j) v_next[j] = (live && j < cnt) ? v[(size_t)(t + j) * ldv + (size_t)h * D + col] : 0.f;
   };
+  auto token = [&](int at, float val, int t) {  // at: where the token's vectors begin in vec
+    const float* wv = vec + at;
+    float d0 = 0.f, d1 = 0.f;
+#pragma unroll
+    for (int j = 0; j < NREG; j += 4) {
+      const float4 u4 = *(const float4*)(wv + 2 * DP + j);
+      d0 = fmaf(S[j], u4.x, d0);
+      d1 = fmaf(S[j + 1], u4.y, d1);
+      d0 = fmaf(S[j + 2], u4.z, d0);
+      d1 = fmaf(S[j + 3], u4.w, d1);
+    }
+    const float dot = groups_sum<COLS>(d0 + d1);  // u^T S_(t-1) of this column
+    float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+    for (int j = 0; j < NREG; j += 4) {
+      const float4 w4 = *(const float4*)(wv + j);
+      const float4 e4 = *(const float4*)(wv + DP + j);
+      const float4 k4 = *(const float4*)(wv + 3 * DP + j);
+      const float4 r4 = *(const float4*)(wv + 4 * DP + j);
+      S[j] = fmaf(w4.x, S[j], fmaf(-e4.x, dot, k4.x * val));
+      a0 = fmaf(S[j], r4.x, a0);
+      S[j + 1] = fmaf(w4.y, S[j + 1], fmaf(-e4.y, dot, k4.y * val));
+      a1 = fmaf(S[j + 1], r4.y, a1);
+      S[j + 2] = fmaf(w4.z, S[j + 2], fmaf(-e4.z, dot, k4.z * val));
+      a0 = fmaf(S[j + 2], r4.z, a0);
+      S[j + 3] = fmaf(w4.w, S[j + 3], fmaf(-e4.w, dot, k4.w * val));
+      a1 = fmaf(S[j + 3], r4.w, a1);
+    }
+    const float acc = groups_sum<COLS>(a0 + a1);
+    if (live && lane < COLS) o[(size_t)t * H * D + (size_t)h * D + col] = acc;
+  };
   ask(t0, n < TB ? n : TB);
   for (int b = 0; b * TB < n; ++b) {
-    const int base = t0 + b * TB, left = n - b * TB, cnt = left < TB ? left : TB;
-    float* blk = vec[b & 1];
+    const int base = t0 + b * TB, left = n - b * TB;
+    const int blk = (b & 1) * TB * TOTAL;
 #pragma unroll
-    for (int u = 0; u < PER; ++u) blk[lane + u * HAL_WAVE] = next[u];
+    for (int u = 0; u < PER; ++u) vec[blk + lane + u * HAL_WAVE] = next[u];
     float vv[TB];
 #pragma unroll
     for (int j = 0; j < TB; ++j) vv[j] = v_next[j];
@@ -147,39 +195,13 @@ delta_scan_kernel(const float* __restrict__ pre, const float* __restrict__ v, in
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    if (left >= TB) {
 #pragma unroll
-    for (int jt = 0; jt < TB; ++jt) {
-      if (jt >= cnt) break;
-      const float* wv = blk + jt * TOTAL + row0;
-      float d0 = 0.f, d1 = 0.f;
+      for (int jt = 0; jt < TB; ++jt) token(blk + jt * TOTAL + row0, vv[jt], base + jt);
+    } else {
 #pragma unroll
-      for (int j = 0; j < NREG; j += 4) {
-        const float4 u4 = *(const float4*)(wv + 2 * DP + j);
-        d0 = fmaf(S[j], u4.x, d0);
-        d1 = fmaf(S[j + 1], u4.y, d1);
-        d0 = fmaf(S[j + 2], u4.z, d0);
-        d1 = fmaf(S[j + 3], u4.w, d1);
-      }
-      const float dot = quarters_sum(d0 + d1);  // u^T S_(t-1) of this column
-      const float val = vv[jt];
-      float a0 = 0.f, a1 = 0.f;
-#pragma unroll
-      for (int j = 0; j < NREG; j += 4) {
-        const float4 w4 = *(const float4*)(wv + j);
-        const float4 e4 = *(const float4*)(wv + DP + j);
-        const float4 k4 = *(const float4*)(wv + 3 * DP + j);
-        const float4 r4 = *(const float4*)(wv + 4 * DP + j);
-        S[j] = fmaf(w4.x, S[j], fmaf(-e4.x, dot, k4.x * val));
-        a0 = fmaf(S[j], r4.x, a0);
-        S[j + 1] = fmaf(w4.y, S[j + 1], fmaf(-e4.y, dot, k4.y * val));
-        a1 = fmaf(S[j + 1], r4.y, a1);
-        S[j + 2] = fmaf(w4.z, S[j + 2], fmaf(-e4.z, dot, k4.z * val));
-        a0 = fmaf(S[j + 2], r4.z, a0);
-        S[j + 3] = fmaf(w4.w, S[j + 3], fmaf(-e4.w, dot, k4.w * val));
-        a1 = fmaf(S[j + 3], r4.w, a1);
-      }
-      const float acc = quarters_sum(a0 + a1);
-      if (live && lane < 16) o[(size_t)(base + jt) * H * D + (size_t)h * D + col] = acc;
+      for (int jt = 0; jt < TB; ++jt)
+        if (jt < left) token(blk + jt * TOTAL + row0, vv[jt], base + jt);
     }
   }
   if (live) {
@@ -190,27 +212,60 @@ delta_scan_kernel(const float* __restrict__ pre, const float* __restrict__ v, in
 }
 
 // ---- a step in which every request brings one token: a workgroup of 256 threads takes one
-// head of one request, reads and writes its state once in rows of 16 bytes a thread (a wave
-// covers whole rows), and the two sums over the key channels cross the waves through LDS.
-// D is 32, 64 or 128; a thread holds R rows of four neighbouring value channels.
+// head of one request.  It reads the state once in rows of 16 bytes a thread (a wave covers
+// whole rows), makes the token's five vectors itself while those loads are on their way
+// (thread c < D a key channel), and the two sums over the key channels cross the waves
+// through LDS.  D is 32, 64 or 128; a thread holds R rows of four neighbouring value channels.
 template <int D>
 __global__ void __launch_bounds__(256)
-delta_step_kernel(const float* __restrict__ pre, const float* __restrict__ v, int ldv, float* __restrict__ state,
-                  const int* __restrict__ token_slot, float* __restrict__ o, int H) {
-  constexpr int CG = D / 4, RG = 256 / CG, R = D / RG, TOTAL = DELTA_VECTORS * D, WAVES = 256 / HAL_WAVE;
+delta_step_kernel(const float* __restrict__ r, int ldr, const float* __restrict__ k, int ldk,
+                  const float* __restrict__ v, int ldv, const float* __restrict__ a_raw, int lda,
+                  const float* __restrict__ x1, int ldx1, const void* __restrict__ w2, const void* __restrict__ w0,
+                  const void* __restrict__ a_bias, int w_dtype, int lora, float decay_rate, float unit_eps,
+                  float* __restrict__ state, const int* __restrict__ token_slot, float* __restrict__ o, int H) {
+  constexpr int CG = D / 4, RG = 256 / CG, R = D / RG, WAVES = 256 / HAL_WAVE;
   static_assert(CG <= HAL_WAVE && 256 % CG == 0 && D % RG == 0, "a head of 32, 64 or 128 channels");
-  __shared__ __align__(16) float vec[TOTAL];
+  __shared__ __align__(16) float vec[DELTA_VECTORS * D];
+  __shared__ float tl[DELTA_MAX_LORA];
+  __shared__ float ksum[WAVES];
   __shared__ float4 red[2][WAVES][CG];
-  const int t = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+  const size_t t = blockIdx.x;
+  const int h = blockIdx.y, tid = threadIdx.x;
   const int cg = tid % CG, rg = tid / CG, col = cg * 4, wave = tid / HAL_WAVE;
-  const float* src = pre + ((size_t)t * H + h) * TOTAL;
-  for (int i = tid; i < TOTAL; i += 256) vec[i] = src[i];
   float* st = state + ((size_t)token_slot[t] * H + h) * D * D + col;
   float4 S[R];
 #pragma unroll
   for (int j = 0; j < R; ++j) S[j] = *(const float4*)(st + (size_t)(rg + j * RG) * D);
-  const float* vr = v + (size_t)t * ldv + (size_t)h * D + col;
+  const float* vr = v + t * ldv + (size_t)h * D + col;
   const float4 vv = make_float4(vr[0], vr[1], vr[2], vr[3]);
+  // the token's vectors
+  const bool channel = tid < D;
+  const size_t ch = (size_t)h * D + (channel ? tid : 0);
+  const float kc = channel ? k[t * ldk + ch] : 0.f;
+  const float ar = channel ? a_raw[t * lda + ch] : 0.f;
+  const float rc = channel ? r[t * ldr + ch] : 0.f;
+  for (int j = tid; j < lora; j += 256) tl[j] = tanhf(x1[t * ldx1 + j]);
+  const float part = wave_sum(kc * kc);
+  if (tid % HAL_WAVE == 0) ksum[wave] = part;
+  __syncthreads();
+  if (channel) {
+    float kk = 0.f;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) kk += ksum[w];
+    float z0 = load_as_f32(w0, w_dtype, ch), z1 = 0.f;
+    int j = 0;
+    for (; j + 1 < lora; j += 2) {
+      z0 = fmaf(load_as_f32(w2, w_dtype, ch * lora + j), tl[j], z0);
+      z1 = fmaf(load_as_f32(w2, w_dtype, ch * lora + j + 1), tl[j + 1], z1);
+    }
+    if (j < lora) z0 = fmaf(load_as_f32(w2, w_dtype, ch * lora + j), tl[j], z0);
+    const float u = kc / sqrtf(kk + unit_eps);
+    vec[tid] = expf(-decay_rate * delta_sigmoid(z0 + z1));
+    vec[D + tid] = delta_sigmoid(ar + load_as_f32(a_bias, w_dtype, ch)) * u;
+    vec[2 * D + tid] = u;
+    vec[3 * D + tid] = kc;
+    vec[4 * D + tid] = rc;
+  }
   __syncthreads();
   auto across = [&](float4 x, int which) {  // the sum over all row groups, in every thread
 #pragma unroll
@@ -241,16 +296,16 @@ delta_step_kernel(const float* __restrict__ pre, const float* __restrict__ v, in
 #pragma unroll
   for (int j = 0; j < R; ++j) {
     const int row = rg + j * RG;
-    const float w = vec[row], e = vec[D + row], k = vec[3 * D + row], r = vec[4 * D + row];
-    S[j].x = fmaf(w, S[j].x, fmaf(-e, dot.x, k * vv.x));
-    S[j].y = fmaf(w, S[j].y, fmaf(-e, dot.y, k * vv.y));
-    S[j].z = fmaf(w, S[j].z, fmaf(-e, dot.z, k * vv.z));
-    S[j].w = fmaf(w, S[j].w, fmaf(-e, dot.w, k * vv.w));
-    acc.x = fmaf(S[j].x, r, acc.x), acc.y = fmaf(S[j].y, r, acc.y), acc.z = fmaf(S[j].z, r, acc.z), acc.w = fmaf(S[j].w, r, acc.w);
+    const float w = vec[row], e = vec[D + row], kr = vec[3 * D + row], rr = vec[4 * D + row];
+    S[j].x = fmaf(w, S[j].x, fmaf(-e, dot.x, kr * vv.x));
+    S[j].y = fmaf(w, S[j].y, fmaf(-e, dot.y, kr * vv.y));
+    S[j].z = fmaf(w, S[j].z, fmaf(-e, dot.z, kr * vv.z));
+    S[j].w = fmaf(w, S[j].w, fmaf(-e, dot.w, kr * vv.w));
+    acc.x = fmaf(S[j].x, rr, acc.x), acc.y = fmaf(S[j].y, rr, acc.y), acc.z = fmaf(S[j].z, rr, acc.z), acc.w = fmaf(S[j].w, rr, acc.w);
     *(float4*)(st + (size_t)row * D) = S[j];
   }
   const float4 out = across(acc, 1);
-  if (tid < CG) *(float4*)(o + (size_t)t * H * D + (size_t)h * D + col) = out;
+  if (tid < CG) *(float4*)(o + t * H * D + (size_t)h * D + col) = out;
 }
 
 // r, k, v, a_raw: float32 [T, H * D] (row-strided views allowed), x1 float32 [T, lora];
@@ -274,29 +329,35 @@ extern "C" int hal_delta_rule(const float* r, int ldr, const float* k, int ldk, 
   HAL_REQUIRE(w_dtype == HAL_F32 || w_dtype == HAL_BF16, "hal_delta_rule: dtype %d", w_dtype);
   if (n_tokens == 0 || n_segs == 0) return 0;
   const int DP = D <= 16 ? 16 : D <= 32 ? 32 : D <= 64 ? 64 : D <= 128 ? 128 : 256;
-  hipLaunchKernelGGL(delta_prep_kernel, dim3((n_tokens + DELTA_PREP_TOKENS - 1) / DELTA_PREP_TOKENS, H),
-                     dim3(DP < 64 ? 64 : DP), 0, stream, r, ldr, k, ldk, a_raw, lda, x1, ldx1, w2, w0, a_bias, w_dtype,
-                     lora, decay_rate, unit_eps, pre, n_tokens, H, D, DP);
-  if (n_tokens == n_segs && (D == 32 || D == 64 || D == 128)) {  // (DP == D for these)
+  if (n_tokens == n_segs && (D == 32 || D == 64 || D == 128)) {
     const dim3 heads(n_tokens, H);
-    if (D == 32)
-      hipLaunchKernelGGL(delta_step_kernel<32>, heads, dim3(256), 0, stream, pre, v, ldv, state, token_slot, o, H);
-    else if (D == 64)
-      hipLaunchKernelGGL(delta_step_kernel<64>, heads, dim3(256), 0, stream, pre, v, ldv, state, token_slot, o, H);
-    else
-      hipLaunchKernelGGL(delta_step_kernel<128>, heads, dim3(256), 0, stream, pre, v, ldv, state, token_slot, o, H);
+#define DELTA_STEP(D_)                                                                                          \
+  hipLaunchKernelGGL(delta_step_kernel<D_>, heads, dim3(256), 0, stream, r, ldr, k, ldk, v, ldv, a_raw, lda, x1, ldx1, \
+                     w2, w0, a_bias, w_dtype, lora, decay_rate, unit_eps, state, token_slot, o, H)
+    if (D == 32) DELTA_STEP(32);
+    else if (D == 64) DELTA_STEP(64);
+    else DELTA_STEP(128);
+#undef DELTA_STEP
     HAL_LAUNCH_CHECK();
     return 0;
   }
-  const dim3 grid(n_segs, H, (D + 15) / 16);
-#define DELTA_SCAN(N_)                                                                                       \
-  hipLaunchKernelGGL(delta_scan_kernel<N_>, grid, dim3(HAL_WAVE), 0, stream, pre, v, ldv, state, seg_q_start, \
-                     seg_q_len, token_slot, o, H, D)
-  if (DP == 16) DELTA_SCAN(4);
-  else if (DP == 32) DELTA_SCAN(8);
-  else if (DP == 64) DELTA_SCAN(16);
-  else if (DP == 128) DELTA_SCAN(32);
-  else DELTA_SCAN(64);
+  // few tokens: a workgroup a token, so that they are made side by side; many: sixteen a
+  // workgroup, which reads its rows of W2 once for all of them
+  if (n_tokens < 256)
+    hipLaunchKernelGGL(delta_prep_kernel<1>, dim3(n_tokens, H), dim3(DP < 64 ? 64 : DP), 0, stream, r, ldr, k, ldk,
+                       a_raw, lda, x1, ldx1, w2, w0, a_bias, w_dtype, lora, decay_rate, unit_eps, pre, n_tokens, H, D, DP);
+  else
+    hipLaunchKernelGGL(delta_prep_kernel<16>, dim3((n_tokens + 15) / 16, H), dim3(DP < 64 ? 64 : DP), 0, stream, r, ldr,
+                       k, ldk, a_raw, lda, x1, ldx1, w2, w0, a_bias, w_dtype, lora, decay_rate, unit_eps, pre, n_tokens, H,
+                       D, DP);
+#define DELTA_SCAN(N_, COLS_)                                                                             \
+  hipLaunchKernelGGL((delta_scan_kernel<N_, COLS_>), dim3(n_segs, H, (D + COLS_ - 1) / COLS_), dim3(HAL_WAVE), 0, \
+                     stream, pre, v, ldv, state, seg_q_start, seg_q_len, token_slot, o, H, D)
+  if (DP == 16) DELTA_SCAN(4, 16);
+  else if (DP == 32) DELTA_SCAN(8, 16);
+  else if (DP == 64) DELTA_SCAN(8, 8);
+  else if (DP == 128) DELTA_SCAN(16, 8);
+  else DELTA_SCAN(32, 8);
 #undef DELTA_SCAN
   HAL_LAUNCH_CHECK();
   return 0;

@@ -151,6 +151,44 @@ def test_delta_rule_in_steps(gpu, stored, shape):
     assert at == T and bool(torch.isnan(state[1]).all()) and bool(torch.isnan(state[3]).all())
 
 
+@pytest.mark.parametrize("shape", [(2, 64, 40), (3, 24, 5), (1, 128, 33)])
+def test_delta_rule_over_a_long_portion(gpu, shape):
+    """Hundreds of tokens in one step (many blocks of the walk, and the kernel that makes the
+    vectors of sixteen tokens at a time, with a rank that is no multiple of its tile) beside a
+    short request, then a step of single tokens on top of the states they left."""
+    H, D, rank = shape
+    n = H * D
+    T = {1: 301, 3: 6}
+    w2, w0, ab = rand(n, rank, seed=1, scale=0.8), rand(n, seed=2, scale=1.5), rand(n, seed=3)
+    rows = {s: rand(t, 4 * n + rank, seed=20 + s) for s, t in T.items()}
+    want = {}
+    for s, a in rows.items():
+        b = a.to(F)
+        r, k, v, a_raw = (b[:, i * n : (i + 1) * n].view(-1, H, D) for i in range(4))
+        x1 = b[:, 4 * n :]
+        decay = torch.exp(-math.exp(-0.5) * torch.sigmoid(torch.tanh(x1) @ w2.to(F).T + w0.to(F))).view(-1, H, D)
+        rate = torch.sigmoid(a_raw + ab.to(F).view(H, D))
+        o = torch.zeros(T[s], H, D, dtype=F)
+        for h in range(H):
+            o[:, h], _ = P.delta_recurrence(r[:, h], k[:, h], v[:, h], decay[:, h], rate[:, h], torch.zeros(D, D, dtype=F))
+        want[s] = o.reshape(T[s], n)
+    state = torch.zeros((4, H, D, D), device=gpu)
+    at = {1: 0, 3: 0}
+    for step in ({1: 300, 3: 5}, {3: 1, 1: 1}):
+        slots = list(step)
+        cuts = [step[s] for s in slots]
+        a = torch.cat([rows[s][at[s] : at[s] + step[s]] for s in slots]).to(gpu)
+        _, starts, lens, slot = step_arrays(gpu, cuts, slots)
+        y = ops.delta_rule(a[:, :n], a[:, n : 2 * n], a[:, 2 * n : 3 * n], a[:, 3 * n : 4 * n], a[:, 4 * n :], w2.to(gpu),
+                           w0.to(gpu), ab.to(gpu), state, starts, lens, slot, math.exp(-0.5), 1e-6).cpu()
+        i = 0
+        for s in slots:
+            ref = want[s][at[s] : at[s] + step[s]]
+            assert float((y[i : i + step[s]] - ref).abs().max()) < 3e-5 * max(1.0, float(want[s].abs().max())), (s, at[s])
+            i += step[s]
+            at[s] += step[s]
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("shape", [(4, 16), (1, 48), (5, 8), (3, 80), (2, 200)])
 def test_norm_weight_and_gate_per_head(gpu, dtype, shape):
