@@ -113,7 +113,8 @@ __device__ __forceinline__ float quarters_sum(float x) {
 // (u^T S and S^T r) cross the groups inside the vector unit.  The tokens' five vectors
 // (shared by the lanes) go through LDS in blocks of TB tokens, the next block's on their way
 // from memory while one is walked, so that the memory's latency is paid once a block and not
-// once a token; a whole block is walked without a branch between its tokens.
+// once a token; a whole block is walked without a branch between its tokens, each token's
+// rows read from LDS while the token before is worked on.
 template <int COLS>
 __device__ __forceinline__ float groups_sum(float x) {
   if (COLS == 8)  // lanes i and i ^ 8: a rotation by 8 inside every row of 16 lanes
@@ -151,33 +152,39 @@ delta_scan_kernel(const float* __restrict__ pre, const float* __restrict__ v, in
 #pragma unroll
     for (int j = 0; j < TB; ++j) v_next[j] = (live && j < cnt) ? v[(size_t)(t + j) * ldv + (size_t)h * D + col] : 0.f;
   };
-  auto token = [&](int at, float val, int t) {  // at: where the token's vectors begin in vec
-    const float* wv = vec + at;
+  // a token's vectors for this lane's rows, read from LDS a token ahead of their use
+  struct Rows { float4 w[NREG / 4], e[NREG / 4], u[NREG / 4], k[NREG / 4], r[NREG / 4]; };
+  auto fetch = [&](Rows& x, int at) {  // at: where the token's vectors begin in vec
+#pragma unroll
+    for (int j = 0; j < NREG / 4; ++j) {
+      x.u[j] = *(const float4*)(vec + at + 2 * DP + 4 * j);
+      x.w[j] = *(const float4*)(vec + at + 4 * j);
+      x.e[j] = *(const float4*)(vec + at + DP + 4 * j);
+      x.k[j] = *(const float4*)(vec + at + 3 * DP + 4 * j);
+      x.r[j] = *(const float4*)(vec + at + 4 * DP + 4 * j);
+    }
+  };
+  auto token = [&](const Rows& x, float val, int t) {
     float d0 = 0.f, d1 = 0.f;
 #pragma unroll
-    for (int j = 0; j < NREG; j += 4) {
-      const float4 u4 = *(const float4*)(wv + 2 * DP + j);
-      d0 = fmaf(S[j], u4.x, d0);
-      d1 = fmaf(S[j + 1], u4.y, d1);
-      d0 = fmaf(S[j + 2], u4.z, d0);
-      d1 = fmaf(S[j + 3], u4.w, d1);
+    for (int j = 0; j < NREG / 4; ++j) {
+      d0 = fmaf(S[4 * j], x.u[j].x, d0);
+      d1 = fmaf(S[4 * j + 1], x.u[j].y, d1);
+      d0 = fmaf(S[4 * j + 2], x.u[j].z, d0);
+      d1 = fmaf(S[4 * j + 3], x.u[j].w, d1);
     }
     const float dot = groups_sum<COLS>(d0 + d1);  // u^T S_(t-1) of this column
     float a0 = 0.f, a1 = 0.f;
 #pragma unroll
-    for (int j = 0; j < NREG; j += 4) {
-      const float4 w4 = *(const float4*)(wv + j);
-      const float4 e4 = *(const float4*)(wv + DP + j);
-      const float4 k4 = *(const float4*)(wv + 3 * DP + j);
-      const float4 r4 = *(const float4*)(wv + 4 * DP + j);
-      S[j] = fmaf(w4.x, S[j], fmaf(-e4.x, dot, k4.x * val));
-      a0 = fmaf(S[j], r4.x, a0);
-      S[j + 1] = fmaf(w4.y, S[j + 1], fmaf(-e4.y, dot, k4.y * val));
-      a1 = fmaf(S[j + 1], r4.y, a1);
-      S[j + 2] = fmaf(w4.z, S[j + 2], fmaf(-e4.z, dot, k4.z * val));
-      a0 = fmaf(S[j + 2], r4.z, a0);
-      S[j + 3] = fmaf(w4.w, S[j + 3], fmaf(-e4.w, dot, k4.w * val));
-      a1 = fmaf(S[j + 3], r4.w, a1);
+    for (int j = 0; j < NREG / 4; ++j) {
+      S[4 * j] = fmaf(x.w[j].x, S[4 * j], fmaf(-x.e[j].x, dot, x.k[j].x * val));
+      a0 = fmaf(S[4 * j], x.r[j].x, a0);
+      S[4 * j + 1] = fmaf(x.w[j].y, S[4 * j + 1], fmaf(-x.e[j].y, dot, x.k[j].y * val));
+      a1 = fmaf(S[4 * j + 1], x.r[j].y, a1);
+      S[4 * j + 2] = fmaf(x.w[j].z, S[4 * j + 2], fmaf(-x.e[j].z, dot, x.k[j].z * val));
+      a0 = fmaf(S[4 * j + 2], x.r[j].z, a0);
+      S[4 * j + 3] = fmaf(x.w[j].w, S[4 * j + 3], fmaf(-x.e[j].w, dot, x.k[j].w * val));
+      a1 = fmaf(S[4 * j + 3], x.r[j].w, a1);
     }
     const float acc = groups_sum<COLS>(a0 + a1);
     if (live && lane < COLS) o[(size_t)t * H * D + (size_t)h * D + col] = acc;
@@ -196,12 +203,23 @@ delta_scan_kernel(const float* __restrict__ pre, const float* __restrict__ v, in
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     if (left >= TB) {
+      Rows cur;
+      fetch(cur, blk + row0);
 #pragma unroll
-      for (int jt = 0; jt < TB; ++jt) token(blk + jt * TOTAL + row0, vv[jt], base + jt);
+      for (int jt = 0; jt < TB; ++jt) {
+        Rows ahead;
+        if (jt + 1 < TB) fetch(ahead, blk + (jt + 1) * TOTAL + row0);
+        token(cur, vv[jt], base + jt);
+        if (jt + 1 < TB) cur = ahead;
+      }
     } else {
 #pragma unroll
       for (int jt = 0; jt < TB; ++jt)
-        if (jt < left) token(blk + jt * TOTAL + row0, vv[jt], base + jt);
+        if (jt < left) {
+          Rows cur;
+          fetch(cur, blk + jt * TOTAL + row0);
+          token(cur, vv[jt], base + jt);
+        }
     }
   }
   if (live) {
