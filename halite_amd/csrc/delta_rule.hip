@@ -19,15 +19,35 @@
 
 __device__ __forceinline__ float delta_sigmoid(float x) { return 1.0f / (1.0f + expf(-x)); }
 
+// sum_j row[j] * x[j] for j < n; `vec`: the row begins at a multiple of four elements
+template <typename W>
+__device__ __forceinline__ float delta_row_dot(const W* __restrict__ row, const float* x, int n, bool vec) {
+  float z0 = 0.f, z1 = 0.f;
+  int j = 0;
+  if (vec) {
+#pragma unroll 4
+    for (; j + 4 <= n; j += 4) {
+      float w[4];
+      load4(row + j, w);
+      z0 = fmaf(w[0], x[j], z0);
+      z1 = fmaf(w[1], x[j + 1], z1);
+      z0 = fmaf(w[2], x[j + 2], z0);
+      z1 = fmaf(w[3], x[j + 3], z1);
+    }
+  }
+  for (; j < n; ++j) z0 = fmaf(to_f32(row[j]), x[j], z0);
+  return z0 + z1;
+}
+
 // ---- a workgroup takes DELTA_PREP_TOKENS tokens of one head; thread c a key channel, whose
 // row of W2 it holds in registers (DELTA_PREP_RANK entries at a time) for all the tokens.
 // pre [T][H][5][DP], zero beyond D.
 #define DELTA_PREP_RANK 32
-template <int DELTA_PREP_TOKENS>
+template <int DELTA_PREP_TOKENS, typename W>
 __global__ void delta_prep_kernel(const float* __restrict__ r, int ldr, const float* __restrict__ k, int ldk,
                                   const float* __restrict__ a_raw, int lda, const float* __restrict__ x1, int ldx1,
-                                  const void* __restrict__ w2, const void* __restrict__ w0,
-                                  const void* __restrict__ a_bias, int w_dtype, int lora, float decay_rate,
+                                  const W* __restrict__ w2, const W* __restrict__ w0,
+                                  const W* __restrict__ a_bias, int lora, float decay_rate,
                                   float unit_eps, float* __restrict__ pre, int n_tokens, int H, int D, int DP) {
   __shared__ float scratch[16];
   __shared__ float tl[DELTA_PREP_TOKENS][DELTA_PREP_RANK];
@@ -37,7 +57,8 @@ __global__ void delta_prep_kernel(const float* __restrict__ r, int ldr, const fl
   const bool live = c < D;
   const size_t ch = (size_t)h * D + (live ? c : 0);
   float z[DELTA_PREP_TOKENS];
-  const float z0 = load_as_f32(w0, w_dtype, ch);
+  const float z0 = to_f32(w0[ch]);
+  const bool vec = lora % 4 == 0;
 #pragma unroll
   for (int i = 0; i < DELTA_PREP_TOKENS; ++i) z[i] = z0;
   for (int j0 = 0; j0 < lora; j0 += DELTA_PREP_RANK) {
@@ -48,8 +69,18 @@ __global__ void delta_prep_kernel(const float* __restrict__ r, int ldr, const fl
       tl[tok][j] = (tok < nt && j < nj) ? tanhf(x1[(size_t)(t0 + tok) * ldx1 + j0 + j]) : 0.f;
     }
     float w[DELTA_PREP_RANK];
+    const W* row = w2 + ch * lora + j0;
+    if (vec && nj == DELTA_PREP_RANK) {
 #pragma unroll
-    for (int j = 0; j < DELTA_PREP_RANK; ++j) w[j] = j < nj ? load_as_f32(w2, w_dtype, ch * lora + j0 + j) : 0.f;
+      for (int j = 0; j < DELTA_PREP_RANK; j += 4) {
+        float q[4];
+        load4(row + j, q);
+        w[j] = q[0], w[j + 1] = q[1], w[j + 2] = q[2], w[j + 3] = q[3];
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < DELTA_PREP_RANK; ++j) w[j] = j < nj ? to_f32(row[j]) : 0.f;
+    }
     __syncthreads();
 #pragma unroll
     for (int i = 0; i < DELTA_PREP_TOKENS; ++i) {
@@ -63,7 +94,7 @@ __global__ void delta_prep_kernel(const float* __restrict__ r, int ldr, const fl
       }
     }
   }
-  const float ab = load_as_f32(a_bias, w_dtype, ch);
+  const float ab = to_f32(a_bias[ch]);
   float kc_[DELTA_PREP_TOKENS], ar_[DELTA_PREP_TOKENS], rc_[DELTA_PREP_TOKENS];
 #pragma unroll
   for (int i = 0; i < DELTA_PREP_TOKENS; ++i) {  // all of a thread's loads on their way at once
@@ -234,17 +265,18 @@ delta_scan_kernel(const float* __restrict__ pre, const float* __restrict__ v, in
 // whole rows), makes the token's five vectors itself while those loads are on their way
 // (thread c < D a key channel), and the two sums over the key channels cross the waves
 // through LDS.  D is 32, 64 or 128; a thread holds R rows of four neighbouring value channels.
-template <int D>
+template <int D, typename W>
 __global__ void __launch_bounds__(256)
 delta_step_kernel(const float* __restrict__ r, int ldr, const float* __restrict__ k, int ldk,
                   const float* __restrict__ v, int ldv, const float* __restrict__ a_raw, int lda,
-                  const float* __restrict__ x1, int ldx1, const void* __restrict__ w2, const void* __restrict__ w0,
-                  const void* __restrict__ a_bias, int w_dtype, int lora, float decay_rate, float unit_eps,
+                  const float* __restrict__ x1, int ldx1, const W* __restrict__ w2, const W* __restrict__ w0,
+                  const W* __restrict__ a_bias, int lora, float decay_rate, float unit_eps,
                   float* __restrict__ state, const int* __restrict__ token_slot, float* __restrict__ o, int H) {
-  constexpr int CG = D / 4, RG = 256 / CG, R = D / RG, WAVES = 256 / HAL_WAVE;
+  constexpr int CG = D / 4, RG = 256 / CG, R = D / RG, WAVES = 256 / HAL_WAVE, PARTS = 256 / D;
   static_assert(CG <= HAL_WAVE && 256 % CG == 0 && D % RG == 0, "a head of 32, 64 or 128 channels");
   __shared__ __align__(16) float vec[DELTA_VECTORS * D];
   __shared__ float tl[DELTA_MAX_LORA];
+  __shared__ float zpart[PARTS][D];
   __shared__ float ksum[WAVES];
   __shared__ float4 red[2][WAVES][CG];
   const size_t t = blockIdx.x;
@@ -266,20 +298,23 @@ delta_step_kernel(const float* __restrict__ r, int ldr, const float* __restrict_
   const float part = wave_sum(kc * kc);
   if (tid % HAL_WAVE == 0) ksum[wave] = part;
   __syncthreads();
+  {  // the decay's sum over the rank, a part of it a thread: thread = (part, channel)
+    const int c = tid % D, part = tid / D;
+    const int per = ((lora + PARTS - 1) / PARTS + 3) & ~3, j0 = part * per;
+    const int n = lora - j0 < per ? lora - j0 : per;
+    zpart[part][c] = n > 0 ? delta_row_dot(w2 + ((size_t)h * D + c) * lora + j0, tl + j0, n, lora % 4 == 0) : 0.f;
+  }
+  __syncthreads();
   if (channel) {
     float kk = 0.f;
 #pragma unroll
     for (int w = 0; w < WAVES; ++w) kk += ksum[w];
-    float z0 = load_as_f32(w0, w_dtype, ch), z1 = 0.f;
-    int j = 0;
-    for (; j + 1 < lora; j += 2) {
-      z0 = fmaf(load_as_f32(w2, w_dtype, ch * lora + j), tl[j], z0);
-      z1 = fmaf(load_as_f32(w2, w_dtype, ch * lora + j + 1), tl[j + 1], z1);
-    }
-    if (j < lora) z0 = fmaf(load_as_f32(w2, w_dtype, ch * lora + j), tl[j], z0);
+    float z = to_f32(w0[ch]);
+#pragma unroll
+    for (int q = 0; q < PARTS; ++q) z += zpart[q][tid];
     const float u = kc / sqrtf(kk + unit_eps);
-    vec[tid] = expf(-decay_rate * delta_sigmoid(z0 + z1));
-    vec[D + tid] = delta_sigmoid(ar + load_as_f32(a_bias, w_dtype, ch)) * u;
+    vec[tid] = expf(-decay_rate * delta_sigmoid(z));
+    vec[D + tid] = delta_sigmoid(ar + to_f32(a_bias[ch])) * u;
     vec[2 * D + tid] = u;
     vec[3 * D + tid] = kc;
     vec[4 * D + tid] = rc;
@@ -349,25 +384,35 @@ extern "C" int hal_delta_rule(const float* r, int ldr, const float* k, int ldk, 
   const int DP = D <= 16 ? 16 : D <= 32 ? 32 : D <= 64 ? 64 : D <= 128 ? 128 : 256;
   if (n_tokens == n_segs && (D == 32 || D == 64 || D == 128)) {
     const dim3 heads(n_tokens, H);
-#define DELTA_STEP(D_)                                                                                          \
-  hipLaunchKernelGGL(delta_step_kernel<D_>, heads, dim3(256), 0, stream, r, ldr, k, ldk, v, ldv, a_raw, lda, x1, ldx1, \
-                     w2, w0, a_bias, w_dtype, lora, decay_rate, unit_eps, state, token_slot, o, H)
-    if (D == 32) DELTA_STEP(32);
-    else if (D == 64) DELTA_STEP(64);
-    else DELTA_STEP(128);
+#define DELTA_STEP(D_, W_)                                                                                          \
+  hipLaunchKernelGGL((delta_step_kernel<D_, W_>), heads, dim3(256), 0, stream, r, ldr, k, ldk, v, ldv, a_raw, lda, x1, \
+                     ldx1, (const W_*)w2, (const W_*)w0, (const W_*)a_bias, lora, decay_rate, unit_eps, state,          \
+                     token_slot, o, H)
+#define DELTA_STEP_OF(W_)         \
+  if (D == 32) DELTA_STEP(32, W_); \
+  else if (D == 64) DELTA_STEP(64, W_); \
+  else DELTA_STEP(128, W_)
+    if (w_dtype == HAL_F32) { DELTA_STEP_OF(float); }
+    else { DELTA_STEP_OF(bf16_t); }
+#undef DELTA_STEP_OF
 #undef DELTA_STEP
     HAL_LAUNCH_CHECK();
     return 0;
   }
   // few tokens: a workgroup a token, so that they are made side by side; many: sixteen a
   // workgroup, which reads its rows of W2 once for all of them
-  if (n_tokens < 256)
-    hipLaunchKernelGGL(delta_prep_kernel<1>, dim3(n_tokens, H), dim3(DP < 64 ? 64 : DP), 0, stream, r, ldr, k, ldk,
-                       a_raw, lda, x1, ldx1, w2, w0, a_bias, w_dtype, lora, decay_rate, unit_eps, pre, n_tokens, H, D, DP);
-  else
-    hipLaunchKernelGGL(delta_prep_kernel<16>, dim3((n_tokens + 15) / 16, H), dim3(DP < 64 ? 64 : DP), 0, stream, r, ldr,
-                       k, ldk, a_raw, lda, x1, ldx1, w2, w0, a_bias, w_dtype, lora, decay_rate, unit_eps, pre, n_tokens, H,
-                       D, DP);
+#define DELTA_PREP(TT_, W_)                                                                                            \
+  hipLaunchKernelGGL((delta_prep_kernel<TT_, W_>), dim3((n_tokens + TT_ - 1) / TT_, H), dim3(DP < 64 ? 64 : DP), 0, stream, \
+                     r, ldr, k, ldk, a_raw, lda, x1, ldx1, (const W_*)w2, (const W_*)w0, (const W_*)a_bias, lora,       \
+                     decay_rate, unit_eps, pre, n_tokens, H, D, DP)
+  if (n_tokens < 256) {
+    if (w_dtype == HAL_F32) DELTA_PREP(1, float);
+    else DELTA_PREP(1, bf16_t);
+  } else {
+    if (w_dtype == HAL_F32) DELTA_PREP(16, float);
+    else DELTA_PREP(16, bf16_t);
+  }
+#undef DELTA_PREP
 #define DELTA_SCAN(N_, COLS_)                                                                             \
   hipLaunchKernelGGL((delta_scan_kernel<N_, COLS_>), dim3(n_segs, H, (D + COLS_ - 1) / COLS_), dim3(HAL_WAVE), 0, \
                      stream, pre, v, ldv, state, seg_q_start, seg_q_len, token_slot, o, H, D)
