@@ -174,14 +174,29 @@ delta_scan_kernel(const float* __restrict__ pre, const float* __restrict__ v, in
   for (int i = 0; i < NREG; ++i) S[i] = (live && row0 + i < D) ? st[(size_t)(row0 + i) * D] : 0.f;
 
   float next[PER], v_next[TB];
+  // where this lane's loads of a block lie from the block's first token on (in floats)
+  int at_pre[PER], tok_pre[PER];
+#pragma unroll
+  for (int u = 0; u < PER; ++u) {
+    const int i = lane + u * HAL_WAVE;
+    tok_pre[u] = i / TOTAL;
+    at_pre[u] = tok_pre[u] * (H * TOTAL - TOTAL) + i;  // token tok_pre[u], entry i - tok_pre[u] * TOTAL
+  }
+  const float* vp = v + (size_t)h * D + (live ? col : 0);
   auto ask = [&](int t, int cnt) {  // tokens t .. t + cnt - 1
+    const float* src = pre + ((size_t)t * H + h) * TOTAL;
+    const float* vs = vp + (size_t)t * ldv;
+    if (cnt == TB) {
 #pragma unroll
-    for (int u = 0; u < PER; ++u) {
-      const int i = lane + u * HAL_WAVE, tok = i / TOTAL;
-      next[u] = tok < cnt ? pre[((size_t)(t + tok) * H + h) * TOTAL + (i - tok * TOTAL)] : 0.f;
+      for (int u = 0; u < PER; ++u) next[u] = src[at_pre[u]];
+#pragma unroll
+      for (int j = 0; j < TB; ++j) v_next[j] = live ? vs[(size_t)j * ldv] : 0.f;
+    } else {
+#pragma unroll
+      for (int u = 0; u < PER; ++u) next[u] = tok_pre[u] < cnt ? src[at_pre[u]] : 0.f;
+#pragma unroll
+      for (int j = 0; j < TB; ++j) v_next[j] = (live && j < cnt) ? vs[(size_t)j * ldv] : 0.f;
     }
-#pragma unroll
-    for (int j = 0; j < TB; ++j) v_next[j] = (live && j < cnt) ? v[(size_t)(t + j) * ldv + (size_t)h * D + col] : 0.f;
   };
   // a token's vectors for this lane's rows, read from LDS a token ahead of their use
   struct Rows { float4 w[NREG / 4], e[NREG / 4], u[NREG / 4], k[NREG / 4], r[NREG / 4]; };
@@ -195,7 +210,10 @@ delta_scan_kernel(const float* __restrict__ pre, const float* __restrict__ v, in
       x.r[j] = *(const float4*)(vec + at + 4 * DP + 4 * j);
     }
   };
-  auto token = [&](const Rows& x, float val, int t) {
+  const bool writer = live && lane < COLS;
+  const size_t o_step = (size_t)H * D;
+  float* op = o + (size_t)t0 * o_step + (size_t)h * D + (live ? col : 0);
+  auto token = [&](const Rows& x, float val) {
     float d0 = 0.f, d1 = 0.f;
 #pragma unroll
     for (int j = 0; j < NREG / 4; ++j) {
@@ -218,7 +236,8 @@ delta_scan_kernel(const float* __restrict__ pre, const float* __restrict__ v, in
       a1 = fmaf(S[4 * j + 3], x.r[j].w, a1);
     }
     const float acc = groups_sum<COLS>(a0 + a1);
-    if (live && lane < COLS) o[(size_t)t * H * D + (size_t)h * D + col] = acc;
+    if (writer) *op = acc;
+    op += o_step;
   };
   ask(t0, n < TB ? n : TB);
   for (int b = 0; b * TB < n; ++b) {
@@ -234,14 +253,14 @@ delta_scan_kernel(const float* __restrict__ pre, const float* __restrict__ v, in
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     if (left >= TB) {
-      Rows cur;
-      fetch(cur, blk + row0);
+      Rows even, odd;  // (TB is even)
+      fetch(even, blk + row0);
 #pragma unroll
-      for (int jt = 0; jt < TB; ++jt) {
-        Rows ahead;
-        if (jt + 1 < TB) fetch(ahead, blk + (jt + 1) * TOTAL + row0);
-        token(cur, vv[jt], base + jt);
-        if (jt + 1 < TB) cur = ahead;
+      for (int jt = 0; jt < TB; jt += 2) {
+        fetch(odd, blk + (jt + 1) * TOTAL + row0);
+        token(even, vv[jt]);
+        if (jt + 2 < TB) fetch(even, blk + (jt + 2) * TOTAL + row0);
+        token(odd, vv[jt + 1]);
       }
     } else {
 #pragma unroll
@@ -249,7 +268,7 @@ delta_scan_kernel(const float* __restrict__ pre, const float* __restrict__ v, in
         if (jt < left) {
           Rows cur;
           fetch(cur, blk + jt * TOTAL + row0);
-          token(cur, vv[jt], base + jt);
+          token(cur, vv[jt]);
         }
     }
   }
