@@ -15,6 +15,7 @@
 #include "hal_api.h"
 
 #define DELTA_MAX_LORA 1024
+#define DELTA_WAVES_FOR_WIDE 4096  // four waves a SIMD of 256 compute units
 #define DELTA_VECTORS 5  // per token and head: decay, a * u, u, k, r
 
 __device__ __forceinline__ float delta_sigmoid(float x) { return 1.0f / (1.0f + expf(-x)); }
@@ -437,6 +438,10 @@ extern "C" int hal_delta_rule(const float* r, int ldr, const float* k, int ldk, 
                      stream, pre, v, ldv, state, seg_q_start, seg_q_len, token_slot, o, H, D)
   if (DP == 16) DELTA_SCAN(4, 16);
   else if (DP == 32) DELTA_SCAN(8, 16);
+  // (eight columns a wave make a token's step short, which is what a lone prompt waits for;
+  // with many waves a SIMD the walk is bound by its LDS reads, and sixteen columns a wave
+  // read half as much for the same part of the state)
+  else if (DP == 64 && (long long)n_segs * H * ((D + 7) / 8) > DELTA_WAVES_FOR_WIDE) DELTA_SCAN(16, 16);
   else if (DP == 64) DELTA_SCAN(8, 8);
   else if (DP == 128) DELTA_SCAN(16, 8);
   else DELTA_SCAN(32, 8);

@@ -189,6 +189,35 @@ def test_delta_rule_over_a_long_portion(gpu, shape):
             at[s] += step[s]
 
 
+def test_delta_rule_over_many_requests(gpu):
+    """So many segments that the walk takes its other layout for heads of 64 (sixteen value
+    channels a wave): 170 requests of 2 to 11 tokens each on states that are not zero."""
+    H, D, rank, R = 4, 64, 8, 170
+    n = H * D
+    w2, w0, ab = rand(n, rank, seed=1, scale=0.8), rand(n, seed=2, scale=1.5), rand(n, seed=3)
+    lens = [2 + (7 * i) % 10 for i in range(R)]
+    a = rand(sum(lens), 4 * n + rank, seed=4)
+    start = 0.3 * rand(R, H, D, D, seed=5)
+    state = start.clone().to(gpu)
+    slots = list(range(R - 1, -1, -1))  # request i lives in slot R - 1 - i
+    _, starts, cuts, slot = step_arrays(gpu, lens, slots)
+    ag = a.to(gpu)
+    y = ops.delta_rule(ag[:, :n], ag[:, n : 2 * n], ag[:, 2 * n : 3 * n], ag[:, 3 * n : 4 * n], ag[:, 4 * n :], w2.to(gpu),
+                       w0.to(gpu), ab.to(gpu), state, starts, cuts, slot, math.exp(-0.5), 1e-6).cpu()
+    left = state.cpu()
+    t0 = 0
+    for i in (0, 1, 57, 168, 169):  # a few of them against the plain recurrence
+        b = a[t0 if i == 0 else sum(lens[:i]) : sum(lens[: i + 1])].to(F)
+        r, k, v, a_raw = (b[:, j * n : (j + 1) * n].view(-1, H, D) for j in range(4))
+        decay = torch.exp(-math.exp(-0.5) * torch.sigmoid(torch.tanh(b[:, 4 * n :]) @ w2.to(F).T + w0.to(F))).view(-1, H, D)
+        rate = torch.sigmoid(a_raw + ab.to(F).view(H, D))
+        for h in range(H):
+            o, S = P.delta_recurrence(r[:, h], k[:, h], v[:, h], decay[:, h], rate[:, h], start[slots[i], h].to(F))
+            got = y[sum(lens[:i]) : sum(lens[: i + 1]), h * D : (h + 1) * D]
+            assert float((got - o).abs().max()) < 3e-5 * max(1.0, float(o.abs().max())), (i, h)
+            assert float((left[slots[i], h] - S).abs().max()) < 3e-5 * max(1.0, float(S.abs().max())), (i, h)
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("shape", [(4, 16), (1, 48), (5, 8), (3, 80), (2, 200)])
 def test_norm_weight_and_gate_per_head(gpu, dtype, shape):
