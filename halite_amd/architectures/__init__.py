@@ -1,3 +1,3 @@
 """Architectures: each module registers itself in ``config.registry`` on import."""
 
-from . import kavuvik, llama, vepitar, zabunex  # noqa: F401
+from . import diporax, kavuvik, llama, vepitar, zabunex  # noqa: F401

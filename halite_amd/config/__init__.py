@@ -1,3 +1,4 @@
+from .diporax import DiporaxConfig
 from .engine import ModelConfig, ServerConfig, parse_overrides
 from .kavuvik import KavuvikConfig
 from .model import Llama3RopeScaling, LlamaConfig
@@ -18,6 +19,7 @@ __all__ = [
     "ARCHITECTURES",
     "Architecture",
     "ConfigError",
+    "DiporaxConfig",
     "KavuvikConfig",
     "LayerRun",
     "LayerSpec",

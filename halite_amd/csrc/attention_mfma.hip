@@ -386,8 +386,20 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
                         j0 >= lo_last[rt];
       // (RULED: sv holds scaled scores, in units of log2, with the bias added)
       const bool far = RULED && p_first[rt] - (j0 + KB - 1) >= rule.bias_len - 1;  // (the same for the wave)
+      // (a capped score: 2 s / cap in units of log2 going in, cap in units of log2 coming out)
+      const float cap_in = RULED && rule.softcap > 0.f ? 2.0f * scale_log2e / rule.softcap : 0.f;
+      const float cap_out = rule.softcap * 1.4426950408889634f;
       auto biased = [&](float raw, int j) {
         if constexpr (RULED) {
+          if (rule.softcap > 0.f) {
+            // cap * tanh(s / cap) = cap * (1 - 2 / (1 + e^(2 s / cap))), in units of log2
+            const float e2 = fast_exp2(raw * cap_in);
+            raw = __builtin_fmaf(-2.0f * cap_out, __builtin_amdgcn_rcpf(1.0f + e2), cap_out);
+            if (rule.bias == nullptr) return raw;
+            int back = p_row[rt] - j;
+            back = back < 0 ? 0 : (back < rule.bias_len ? back : rule.bias_len - 1);
+            return raw + rule.bias[(size_t)head[rt] * rule.bias_len + back];
+          }
           if (rule.bias == nullptr) return raw * scale_log2e;
           if (far) return __builtin_fmaf(raw, scale_log2e, far_bias[rt]);
           int back = p_row[rt] - j;
@@ -887,7 +899,8 @@ attention_mfma_kernel(const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __
     if (!row_ok[rt]) continue;
     if (partial < 0 || merged_here) {
       if constexpr (RULED) {
-        if (rule.sink == HAL_WEIGHTS_SINK && m[rt] != -INFINITY) lt += exp2f(-m[rt]);  // (sums are relative to 2^m)
+        if (rule.sink == HAL_WEIGHTS_SINK && m[rt] != -INFINITY)  // (sums are relative to 2^m)
+          lt += exp2f((rule.sink_value ? rule.sink_value[head[rt]] : 0.f) - m[rt]);
       }
       float inv = lt > 0.f ? 1.0f / lt : 0.f;
       if constexpr (RULED) {
@@ -924,7 +937,7 @@ __global__ void __launch_bounds__(256)
 attention_merge_kernel(bf16_t* __restrict__ out, int out_row_stride,
                        const int* __restrict__ merges, const int* __restrict__ n_merges_ptr,
                        const float* __restrict__ part_o, const float* __restrict__ part_ml, int H,
-                       int K, int sink) {
+                       int K, int sink, const float* __restrict__ sink_log2) {
   constexpr int NC = (D + 127) / 128;  // a lane's pairs of dimensions
   constexpr int MW = 4;                // waves
   __shared__ float red_o[MW][NC * 128];
@@ -996,10 +1009,10 @@ attention_merge_kernel(bf16_t* __restrict__ out, int out_row_stride,
   float l_sum = 0.f;
 #pragma unroll
   for (int w = 0; w < MW; ++w) l_sum += red_l[w];
-  if (sink == HAL_WEIGHTS_SINK && m_all != -INFINITY) l_sum += exp2f(-m_all);
+  const int qi = rho / G, head = g * G + rho % G;
+  if (sink == HAL_WEIGHTS_SINK && m_all != -INFINITY) l_sum += exp2f((sink_log2 ? sink_log2[head] : 0.f) - m_all);
   float inv = l_sum > 0.f ? 1.0f / l_sum : 0.f;
   if (sink == HAL_WEIGHTS_SIGMOID) inv = m_all != -INFINITY ? exp2f(m_all) : 0.f;
-  const int qi = rho / G, head = g * G + rho % G;
   bf16_t* op = out + (size_t)(q_start + qi) * out_row_stride + (size_t)head * D;
 #pragma unroll
   for (int c = 0; c < NC; ++c) {
@@ -1022,7 +1035,7 @@ __global__ void __launch_bounds__(256)
 attention_merge_few_kernel(bf16_t* __restrict__ out, int out_row_stride,
                            const int* __restrict__ merges, const int* __restrict__ n_merges_ptr,
                            const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                           int H, int K, int sink) {
+                           int H, int K, int sink, const float* __restrict__ sink_log2) {
   constexpr int NC = (D + 127) / 128;
   const int mi = blockIdx.x;
   const int lane = threadIdx.x % HAL_WAVE, wave = threadIdx.x / HAL_WAVE;
@@ -1054,10 +1067,10 @@ attention_merge_few_kernel(bf16_t* __restrict__ out, int out_row_stride,
       acc[c][1] += w * v.y;
     }
   }
-  if (sink == HAL_WEIGHTS_SINK && m_all != -INFINITY) l_all += exp2f(-m_all);
+  const int qi = rho / G, head = g * G + rho % G;
+  if (sink == HAL_WEIGHTS_SINK && m_all != -INFINITY) l_all += exp2f((sink_log2 ? sink_log2[head] : 0.f) - m_all);
   float inv = l_all > 0.f ? 1.0f / l_all : 0.f;
   if (sink == HAL_WEIGHTS_SIGMOID) inv = m_all != -INFINITY ? exp2f(m_all) : 0.f;
-  const int qi = rho / G, head = g * G + rho % G;
   bf16_t* op = out + (size_t)(q_start + qi) * out_row_stride + (size_t)head * D;
 #pragma unroll
   for (int c = 0; c < NC; ++c) {
@@ -1110,7 +1123,7 @@ extern "C" int hal_attention_mfma(const void* q, int q_row_stride, void* out, in
                                   max_big, merges, max_merges, counts, seg_q_start, seg_q_len,
                                   seg_kv_len, block_table, bt_stride, k_pages, v_pages, part_o, part_ml,
                                   counters, n_counters, H, K, head_dim, page_size, tiled, scale, window,
-                                  0, nullptr, 0, 0, merge_parts, stream);
+                                  0, nullptr, 0, 0, 0.f, nullptr, merge_parts, stream);
 }
 
 // The same with a rule for the scores.  `chunk`: the work lists must have been cut for it (a
@@ -1126,12 +1139,15 @@ extern "C" int hal_attention_mfma_ruled(const void* q, int q_row_stride, void* o
                                         int* counters, int n_counters, int H, int K, int head_dim,
                                         int page_size, int tiled, float scale, int window, int chunk,
                                         const float* bias_log2, int bias_len, int sink,
+                                        float softcap, const float* sink_log2,
                                         int merge_parts, hipStream_t stream) {
   HAL_REQUIRE(chunk >= 0 && (bias_log2 == nullptr || bias_len > 0),
               "hal_attention_mfma: chunk %d, bias table of %d distances", chunk, bias_len);
   HAL_REQUIRE(sink >= HAL_WEIGHTS_SOFTMAX && sink <= HAL_WEIGHTS_SIGMOID, "hal_attention_mfma: weights of kind %d", sink);
-  const hal_score_rule rule = {window, chunk, bias_len, sink, bias_log2};
-  const bool ruled = bias_log2 != nullptr || sink;
+  HAL_REQUIRE(softcap >= 0.f && (sink_log2 == nullptr || sink == HAL_WEIGHTS_SINK),
+              "hal_attention_mfma: a cap of %g, or sink values without a sink", (double)softcap);
+  const hal_score_rule rule = {window, chunk, bias_len, sink, bias_log2, softcap, sink_log2};
+  const bool ruled = bias_log2 != nullptr || sink || softcap > 0.f;
   HAL_REQUIRE(head_dim == D, "hal_attention_mfma: built for head size %d, called with %d", D,
               head_dim);
   HAL_REQUIRE(H > 0 && K > 0 && H % K == 0, "hal_attention_mfma: %d heads, %d kv heads", H, K);
@@ -1183,11 +1199,11 @@ extern "C" int hal_attention_mfma_ruled(const void* q, int q_row_stride, void* o
     if (merge_parts > 0 && merge_parts <= MERGE_FEW_PARTS)
       hipLaunchKernelGGL(attention_merge_few_kernel, dim3(max_merges, K, 4), dim3(256), 0, stream,
                          (bf16_t*)out, out_row_stride, merges, counts + 2, part_o, part_ml, H, K,
-                         rule.sink);
+                         rule.sink, rule.sink_value);
     else
       hipLaunchKernelGGL(attention_merge_kernel, dim3(max_merges, K, 16), dim3(256), 0, stream,
                          (bf16_t*)out, out_row_stride, merges, counts + 2, part_o, part_ml, H, K,
-                         rule.sink);
+                         rule.sink, rule.sink_value);
     HAL_LAUNCH_CHECK();
   }
   return 0;

@@ -354,7 +354,7 @@ attention_plain_kernel(const T* __restrict__ q, int q_row_stride, T* __restrict_
               plain_swap_32(dot, other);  // (one of the two is this lane's, the other its partner's)
               dot = dot + other;
             }
-            if (valid) s = dot * scale;
+            if (valid) s = hal_rule_cap(rule, dot * scale);
             if (valid && rule.bias) s += hal_rule_bias(rule, h_first + r % heads_here, p - j);
             if (valid && rule.sink == HAL_WEIGHTS_SIGMOID) s = hal_log_sigmoid(s);
           }
@@ -428,7 +428,7 @@ attention_plain_kernel(const T* __restrict__ q, int q_row_stride, T* __restrict_
       const bool only_piece = (lo >> piece_shift) == (p >> piece_shift);
       if (r >= n_rows || (split && !(only_piece && blockIdx.z == 0))) continue;
       T* op = out + (size_t)(ta + r / heads_here) * out_row_stride + (size_t)(h_first + r % heads_here) * D;
-      const float inv = hal_rule_inverse(rule, M[rr], L[rr]);
+      const float inv = hal_rule_inverse(rule, M[rr], L[rr], h_first + r % heads_here);
 #pragma unroll
       for (int c = 0; c < R; ++c) {
         const int d = lane + c * HAL_WAVE;
@@ -482,7 +482,7 @@ attention_plain_merge_kernel(T* __restrict__ out, int out_row_stride, const int*
     }
   }
   T* op = out + (size_t)t * out_row_stride + (size_t)h * D;
-  const float inv = hal_rule_inverse(rule, M, L);
+  const float inv = hal_rule_inverse(rule, M, L, h);
 #pragma unroll
   for (int c = 0; c < R; ++c) {
     const int d = lane + c * HAL_WAVE;
@@ -637,7 +637,7 @@ attention_rows_kernel(const T* __restrict__ q, int q_row_stride, T* __restrict__
       for (int v = 0; v < 16; ++v) {
         const int j = j0 + 8 * (v / 4) + 4 * half + v % 4;
         valid[v] = j >= lo && j <= p;
-        st[v] = valid[v] ? st[v] * scale + (rule.bias ? hal_rule_bias(rule, head, p - j) : 0.f) : -INFINITY;
+        st[v] = valid[v] ? hal_rule_cap(rule, st[v] * scale) + (rule.bias ? hal_rule_bias(rule, head, p - j) : 0.f) : -INFINITY;
         if (valid[v] && rule.sink == HAL_WEIGHTS_SIGMOID) st[v] = hal_log_sigmoid(st[v]);
         mx = fmaxf(mx, st[v]);
       }
@@ -681,7 +681,7 @@ attention_rows_kernel(const T* __restrict__ q, int q_row_stride, T* __restrict__
     }
     if (have_row) {  // element v of a block's 16: dimension 32 b + 8 (v / 4) + 4 half + v % 4
       T* op = out + (size_t)token * out_row_stride + (size_t)head * D;
-      const float inv = hal_rule_inverse(rule, m, l);
+      const float inv = hal_rule_inverse(rule, m, l, head);
 #pragma unroll
       for (int b = 0; b < DB; ++b)
 #pragma unroll
@@ -755,8 +755,8 @@ extern "C" int hal_attention_simple(const void* q, int q_row_stride, void* out,
                                     hipStream_t stream) {
   return hal_attention_simple_ruled(q, q_row_stride, out, out_row_stride, dtype, positions, token_seg,
                                     block_table, bt_stride, k_pages, v_pages, part, n_tokens, H, K, D,
-                                    page_size, n_pages, scale, window, 0, nullptr, 0, 0, max_kv_len,
-                                    min_q_len, stream);
+                                    page_size, n_pages, scale, window, 0, nullptr, 0, 0, 0.f, nullptr,
+                                    max_kv_len, min_q_len, stream);
 }
 
 extern "C" int hal_attention_simple_ruled(const void* q, int q_row_stride, void* out,
@@ -765,12 +765,15 @@ extern "C" int hal_attention_simple_ruled(const void* q, int q_row_stride, void*
                                           const void* k_pages, const void* v_pages, float* part,
                                           int n_tokens, int H, int K, int D, int page_size, int n_pages,
                                           float scale, int window, int chunk, const float* bias,
-                                          int bias_len, int sink, int max_kv_len, int min_q_len,
+                                          int bias_len, int sink, float softcap,
+                                          const float* sink_value, int max_kv_len, int min_q_len,
                                           hipStream_t stream) {
   HAL_REQUIRE(chunk >= 0 && (bias == nullptr || bias_len > 0),
               "hal_attention_simple: chunk %d, bias table of %d distances", chunk, bias_len);
   HAL_REQUIRE(sink >= HAL_WEIGHTS_SOFTMAX && sink <= HAL_WEIGHTS_SIGMOID, "hal_attention_simple: weights of kind %d", sink);
-  const hal_score_rule rule = {window, chunk, bias_len, sink, bias};
+  HAL_REQUIRE(softcap >= 0.f && (sink_value == nullptr || sink == HAL_WEIGHTS_SINK),
+              "hal_attention_simple: a cap of %g, or sink values without a sink", (double)softcap);
+  const hal_score_rule rule = {window, chunk, bias_len, sink, bias, softcap, sink_value};
   HAL_REQUIRE(n_tokens >= 0 && H > 0 && K > 0 && D > 0 && page_size > 0 && n_pages > 0,
               "hal_attention_simple: bad sizes T=%d H=%d K=%d D=%d page=%d pages=%d", n_tokens, H,
               K, D, page_size, n_pages);

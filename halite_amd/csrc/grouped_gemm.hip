@@ -33,7 +33,8 @@ struct GroupedArgs {
   const int* row_dst;  // or null
   const float* gate;   // or null
   int ldg;
-  float limit, alpha;
+  int gate_group_cols, gate_cols;  // the gate of group g, column n: gate[row][g * gate_group_cols + (gate_cols ? n : 0)]
+  float limit, alpha, up_shift;
   int act;  // without W2: 0 the product as it is, 1 the square of its positive part
 };
 
@@ -70,7 +71,7 @@ __device__ __forceinline__ void gg_store(const GroupedArgs& a, int g, int i, int
   if (gated) {
     const float gg = fminf(v, a.limit);
     const float uu = fminf(fmaxf(v2, -a.limit), a.limit);
-    v = gg * gg_sigmoid(a.alpha * gg) * (uu + 1.0f);
+    v = gg * gg_sigmoid(a.alpha * gg) * (uu + a.up_shift);
   }
   if (!gated && a.act == 1) {
     v = fmaxf(v, 0.f);
@@ -78,7 +79,7 @@ __device__ __forceinline__ void gg_store(const GroupedArgs& a, int g, int i, int
   }
   const int dst = a.row_dst ? a.row_dst[i] : i;
   const size_t col = (size_t)g * a.y_group_cols + a.y_col0 + n;
-  if (a.gate) v *= gg_sigmoid(a.gate[(size_t)dst * a.ldg + (size_t)g * a.y_group_cols + n]);
+  if (a.gate) v *= gg_sigmoid(a.gate[(size_t)dst * a.ldg + (size_t)g * a.gate_group_cols + (a.gate_cols ? n : 0)]);
   const size_t at = (size_t)dst * a.ldy + col;
   if (a.y_dtype == HAL_F32) {
     float* y = (float*)a.Y;
@@ -359,7 +360,8 @@ extern "C" int hal_grouped_gemm(const void* X, int ldx, int x_group_cols, int x_
                                 void* Y, int ldy, int y_group_cols, int y_col0, int y_dtype,
                                 int y_add, int M, int N, int K, int G, const int* group_offsets,
                                 const int* tile_offsets, const int* row_src, int src_div,
-                                const int* row_dst, const float* gate, int ldg, float limit,
+                                const int* row_dst, const float* gate, int ldg, int gate_per_group,
+                                float limit, float up_shift,
                                 float alpha, int act, int allow_mfma, hipStream_t stream) {
   HAL_REQUIRE(act == 0 || (act == 1 && W2 == nullptr), "hal_grouped_gemm: activation %d", act);
   HAL_REQUIRE(M >= 0 && N > 0 && K > 0 && G > 0, "hal_grouped_gemm: bad sizes M=%d N=%d K=%d G=%d", M, N,
@@ -380,7 +382,9 @@ extern "C" int hal_grouped_gemm(const void* X, int ldx, int x_group_cols, int x_
   a.M = M; a.N = N; a.K = K; a.G = G;
   a.group_offsets = group_offsets; a.tile_offsets = tile_offsets;
   a.row_src = row_src; a.src_div = src_div; a.row_dst = row_dst;
-  a.gate = gate; a.ldg = ldg; a.limit = limit; a.alpha = alpha; a.act = act;
+  a.gate = gate; a.ldg = ldg; a.limit = limit; a.alpha = alpha; a.act = act; a.up_shift = up_shift;
+  a.gate_group_cols = gate_per_group ? 1 : y_group_cols;
+  a.gate_cols = gate_per_group ? 0 : 1;
   const int row_tiles = (M + GG_ROWS - 1) / GG_ROWS;
   // (a list of M rows cut into G groups has at most M / tile + G tiles, each group's last one partly filled)
   dim3 grid((N + GG_TN - 1) / GG_TN * (GG_ROWS / GG_TM), group_offsets ? row_tiles + G : row_tiles,

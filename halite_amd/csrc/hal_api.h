@@ -56,14 +56,17 @@ int hal_attention_simple(const void* q, int q_row_stride, void* out, int out_row
 // hal_attention_simple with a rule for the scores: `chunk` > 0: a query sees no key before
 // the start of its own chunk of that many positions; `bias` (or null): float32
 // [H][bias_len], added to the scaled score of the key n tokens back at
-// [head][min(n, bias_len - 1)]; `sink`: one more term of score 0 and no value in the softmax.
+// [head][min(n, bias_len - 1)]; `sink`: one more term of score 0 and no value in the softmax
+// (`sink_value`, or null: float32 [H], that term's score per head instead of 0); `softcap` > 0:
+// the scaled score s becomes softcap * tanh(s / softcap) before the bias.
 int hal_attention_simple_ruled(const void* q, int q_row_stride, void* out, int out_row_stride,
                                int dtype, const int* positions, const int* token_seg,
                                const int* block_table, int bt_stride, const void* k_pages,
                                const void* v_pages, float* part, int n_tokens, int H, int K, int D,
                                int page_size, int n_pages, float scale, int window, int chunk,
-                               const float* bias, int bias_len, int sink, int max_kv_len,
-                               int min_q_len, hipStream_t stream);
+                               const float* bias, int bias_len, int sink, float softcap,
+                               const float* sink_value, int max_kv_len, int min_q_len,
+                               hipStream_t stream);
 
 int hal_gemm_f32(const float* A, int lda, const float* W, int ldw, float* C, int ldc, int M,
                  int N, int K, hipStream_t stream);
@@ -148,8 +151,9 @@ int hal_grouped_gemm(const void* X, int ldx, int x_group_cols, int x_col0, const
                      const void* W2, long long w_group_stride, int ldw, int dtype, void* Y, int ldy,
                      int y_group_cols, int y_col0, int y_dtype, int y_add, int M, int N, int K,
                      int G, const int* group_offsets, const int* tile_offsets, const int* row_src,
-                     int src_div, const int* row_dst, const float* gate, int ldg, float limit,
-                     float alpha, int act, int allow_mfma, hipStream_t stream);
+                     int src_div, const int* row_dst, const float* gate, int ldg, int gate_per_group,
+                     float limit, float up_shift, float alpha, int act, int allow_mfma,
+                     hipStream_t stream);
 
 // ---- around a latent attention and a mixture of experts (latent_moe.hip) -----------------
 // RMSNorm of rows of the float32 stream (rows[r] or r) with one or two weights, x * rstd * w
@@ -174,21 +178,22 @@ int hal_scale_f32(float* x, long long n, float s, hipStream_t stream);
 // Router of a mixture of experts on float32 logits z [T, E]: scores by sigmoid (softmax over
 // the experts if `softmax`), the `top` largest (lower index on a tie) to idx [T, top], their
 // scores (divided by their sum + norm_eps if `normalize`) to wgt [T, top].
-int hal_moe_route(const float* z, int E, int top, int softmax, int normalize, float norm_eps,
+int hal_moe_route(const float* z, int ldz, int E, int top, int softmax, int normalize, float norm_eps,
                   int* idx, float* wgt, int n_tokens, hipStream_t stream);
 // Counting sort of the n (token, choice) pairs by expert (idx [n]); offsets, tile_offsets
 // [E + 1] and sorted [n] as hal_grouped_gemm takes them (tiles of `tile` rows).
 int hal_moe_sort(const int* idx, int n, int E, int tile, int* offsets, int* tile_offsets,
                  int* sorted, hipStream_t stream);
-// h[t] += sum_j wgt[t, j] * y[t * top + j] (+ extra[t] if given)  (h, extra [T, d] and
-// y [T * top, d] float32)
-int hal_moe_combine(float* h, const float* y, const float* wgt, const float* extra, int top, int d,
-                    int n_tokens, hipStream_t stream);
+// h[t] += sum_j wgt[t, j] * y[t * top + j] (+ extra[t] if given, times sigmoid(extra_gate[t *
+// ld_gate]) if that is given)  (h, extra [T, d] and y [T * top, d] float32)
+int hal_moe_combine(float* h, const float* y, const float* wgt, const float* extra,
+                    const float* extra_gate, int ld_gate, int top, int d, int n_tokens,
+                    hipStream_t stream);
 
-// out [T, F] = g * sigmoid(alpha * g) * (u + 1), g = min(gu[t, f], limit), u = clamp(gu[t, F + f],
+// out [T, F] = g * sigmoid(alpha * g) * (u + up_shift), g = min(gu[t, f], limit), u = clamp(gu[t, F + f],
 // -limit, limit), for rows gu [T, 2F] that hold a gate projection and an up projection.
 int hal_clamped_gate_mul(const void* gu, void* out, int dtype, int n_tokens, int F, float limit,
-                         float alpha, hipStream_t stream);
+                         float alpha, float up_shift, hipStream_t stream);
 
 // ---- rows of the stream and of projections (stream_ops.hip) -------------------------------
 // out = T(h), n elements
@@ -237,12 +242,14 @@ int hal_short_conv_carry(const float* u, int ldu, float* state, int taps, const 
 // y [T, heads * P] float32 = S_t^T C_t + D x_t.  chunks [n_chunks][4] (first token, tokens,
 // segment, 0), seg_chunks [segments][2] (first chunk, chunks), sums (n_chunks * heads * N * P
 // floats) and decays (n_chunks * heads floats): the segments cut into chunks that are walked
-// side by side, or all null: a wave walks a whole segment.
+// side by side, or all null: a wave walks a whole segment.  fixed_decay (or null): float32
+// [heads], one constant decay a head with step sizes of 1 and no D: S <- decay S + B x^T.
 int hal_ssd_scan(const void* xbc, int ldx, int dtype, const float* dt_raw, int ld_dt,
                  const void* dt_bias, const void* a_log, const void* d_skip, int w_dtype,
                  float* state, const int* seg_q_start, const int* seg_q_len, const int* token_slot,
                  float* y, int n_segs, int heads, int P, int N, int groups, const int* chunks,
-                 const int* seg_chunks, int n_chunks, float* sums, float* decays, hipStream_t stream);
+                 const int* seg_chunks, int n_chunks, float* sums, float* decays,
+                 const float* fixed_decay, hipStream_t stream);
 // out = (y * silu(z)) / rms over each of `parts` equal parts of the row * w
 int hal_gated_part_norm(const float* y, const float* z, int ldz, const void* w, int w_dtype,
                         float eps, void* out, int dtype, int n_tokens, int inner, int parts,
@@ -277,11 +284,21 @@ int hal_streams_step(float* x, long long copy_stride, int S, const float* y, con
                      int result_dtype, const int* rows, int n_rows, int W, hipStream_t stream);
 // Every head of float32 q [T, H * dq], k [T, K * dq], v [T, K * dv] divided by its own root
 // mean square, packed as hal_qk_norm_pack packs (and appended to the pages, if given).
+// w_q, w_k (or null): a weight [dq] for every normed head of q / k; norm_v 0: the values are not
+// divided; v_other (or null): the values become (1 - v_mix) v + v_mix v_other.
 int hal_head_norm_pack(const float* q, int ldq, const float* k, int ldk, const float* v, int ldv, float eps,
-                       const int* positions, void* out, int row_stride, int dtype, int n_tokens, int H,
+                       const void* w_q, const void* w_k, int w_dtype, int norm_v, const float* v_other,
+                       int ldvo, float v_mix, const int* positions, void* out, int row_stride, int dtype, int n_tokens, int H,
                        int K, int dq, int dv, int D, const int* token_seg, const int* block_table,
                        int bt_stride, void* k_pages, void* v_pages, int page_size, int n_pages, int tiled,
                        hipStream_t stream);
+// a[t, c] += bias[c] (float32 rows, in place)
+int hal_bias_rows(float* a, int lda, const void* bias, int b_dtype, int n_rows, int n_cols, hipStream_t stream);
+// out[t, c] = silu(a[t, c]) for the first n_cols columns of float32 rows
+int hal_silu_rows(const float* a, int lda, void* out, int dtype, int n_rows, int n_cols, hipStream_t stream);
+// out[t, j] = gelu_tanh(g[t, j]) * table[tokens[t]][col0 + j], j < dim (a token out of range: NaN)
+int hal_token_gate(const float* g, int ldg, const void* table, int t_dtype, int ld_table, int col0,
+                   const int* tokens, int vocab, void* out, int dtype, int n_rows, int dim, hipStream_t stream);
 // y[t, h * n + j] = x[t, h * x_head + j] * sigmoid(g[t, h]), j < n
 int hal_head_gate_cols(const void* x, int ldx, int x_head, const float* g, int ldg, void* y, int n, int H,
                        int dtype, int n_tokens, hipStream_t stream);
@@ -306,7 +323,7 @@ int hal_attention_mfma(const void* q, int q_row_stride, void* out, int out_row_s
                        float scale, int window, int merge_parts, hipStream_t stream);
 
 // hal_attention_mfma with a rule for the scores (see hal_attention_simple_ruled); the bias
-// table comes multiplied by log2 e, and the work lists are cut for the chunk.
+// table and the sinks' values come multiplied by log2 e, and the work lists are cut for the chunk.
 int hal_attention_mfma_ruled(const void* q, int q_row_stride, void* out, int out_row_stride,
                              const int* items, int max_items, const int* big_items, int max_big,
                              const int* merges, int max_merges, const int* counts,
@@ -315,6 +332,7 @@ int hal_attention_mfma_ruled(const void* q, int q_row_stride, void* out, int out
                              const void* v_pages, float* part_o, float* part_ml, int* counters,
                              int n_counters, int H, int K, int head_dim, int page_size, int tiled,
                              float scale, int window, int chunk, const float* bias_log2,
-                             int bias_len, int sink, int merge_parts, hipStream_t stream);
+                             int bias_len, int sink, float softcap, const float* sink_log2,
+                             int merge_parts, hipStream_t stream);
 
 }  // extern "C"

@@ -148,7 +148,9 @@ __host__ __device__ __forceinline__ size_t kv_value_offset(bool tiled, int page_
 // weight is the sigmoid of its score (scaled, bias added) and the weights are not normalised
 // over the keys.  The kernels keep their sums relative to a running maximum m either way: they
 // are handed the logarithm of the sigmoid as the score, and a finished row is multiplied by
-// exp(m) where a softmax's is divided by its sum.
+// exp(m) where a softmax's is divided by its sum.  `softcap` > 0: the scaled score s becomes
+// softcap * tanh(s / softcap) before anything is added to it.  `sink_value` (or null, with
+// HAL_WEIGHTS_SINK): float32 [heads], the score of the sink's term of every head instead of 0.
 enum { HAL_WEIGHTS_SOFTMAX = 0, HAL_WEIGHTS_SINK = 1, HAL_WEIGHTS_SIGMOID = 2 };
 struct hal_score_rule {
   int window;
@@ -156,6 +158,8 @@ struct hal_score_rule {
   int bias_len;
   int sink;
   const float* bias;
+  float softcap;
+  const float* sink_value;
 };
 __host__ __device__ __forceinline__ int hal_rule_lo(const hal_score_rule& r, int p) {
   int lo = 0;
@@ -168,9 +172,13 @@ __device__ __forceinline__ float hal_rule_bias(const hal_score_rule& r, int head
 }
 // what a finished row's sums (taken relative to the maximum m) are multiplied by:
 // 1 / (l + the sink's term), or exp(m) for weights that are not normalised
-__device__ __forceinline__ float hal_rule_inverse(const hal_score_rule& r, float m, float l) {
+__device__ __forceinline__ float hal_rule_inverse(const hal_score_rule& r, float m, float l, int head) {
   if (r.sink == HAL_WEIGHTS_SIGMOID) return expf(m);
-  return 1.0f / (r.sink == HAL_WEIGHTS_SINK ? l + expf(-m) : l);
+  if (r.sink != HAL_WEIGHTS_SINK) return 1.0f / l;
+  return 1.0f / (l + expf((r.sink_value ? r.sink_value[head] : 0.f) - m));
+}
+__device__ __forceinline__ float hal_rule_cap(const hal_score_rule& r, float s) {
+  return r.softcap > 0.f ? r.softcap * tanhf(s / r.softcap) : s;
 }
 // ln sigmoid(s) = min(s, 0) - ln(1 + exp(-|s|))
 __device__ __forceinline__ float hal_log_sigmoid(float s) {

@@ -184,11 +184,11 @@ extern "C" int hal_scale_f32(float* x, long long n, float s, hipStream_t stream)
 // One wave a token: lane l holds the scores of the experts l, l + 64, ...; each of the `top`
 // rounds finds the largest score that is left (the lower index on a tie) across the wave.
 #define MOE_ROUTE_PER_LANE (MOE_MAX_EXPERTS / HAL_WAVE)
-__global__ void __launch_bounds__(HAL_WAVE) moe_route_kernel(const float* __restrict__ z, int E, int top, int softmax,
+__global__ void __launch_bounds__(HAL_WAVE) moe_route_kernel(const float* __restrict__ z, int ldz, int E, int top, int softmax,
                                                              int normalize, float norm_eps, int* __restrict__ idx,
                                                              float* __restrict__ wgt, int n_tokens) {
   const int t = blockIdx.x, lane = threadIdx.x;
-  const float* zr = z + (size_t)t * E;
+  const float* zr = z + (size_t)t * ldz;
   float s[MOE_ROUTE_PER_LANE];
   float zmax = -INFINITY;
 #pragma unroll
@@ -243,13 +243,13 @@ __global__ void __launch_bounds__(HAL_WAVE) moe_route_kernel(const float* __rest
   }
 }
 
-extern "C" int hal_moe_route(const float* z, int E, int top, int softmax, int normalize,
+extern "C" int hal_moe_route(const float* z, int ldz, int E, int top, int softmax, int normalize,
                              float norm_eps, int* idx, float* wgt, int n_tokens,
                              hipStream_t stream) {
-  HAL_REQUIRE(n_tokens >= 0 && E > 0 && E <= MOE_MAX_EXPERTS && top > 0 && top <= E,
+  HAL_REQUIRE(n_tokens >= 0 && E > 0 && E <= MOE_MAX_EXPERTS && top > 0 && top <= E && ldz >= E,
               "hal_moe_route: bad sizes T=%d E=%d top=%d", n_tokens, E, top);
   if (n_tokens == 0) return 0;
-  hipLaunchKernelGGL(moe_route_kernel, dim3(n_tokens), dim3(HAL_WAVE), 0, stream, z, E, top, softmax,
+  hipLaunchKernelGGL(moe_route_kernel, dim3(n_tokens), dim3(HAL_WAVE), 0, stream, z, ldz, E, top, softmax,
                      normalize, norm_eps, idx, wgt, n_tokens);
   HAL_LAUNCH_CHECK();
   return 0;
@@ -307,23 +307,25 @@ extern "C" int hal_moe_sort(const int* idx, int n, int E, int tile, int* offsets
 // h[t, :] += sum_j wgt[t, j] * y[t * top + j, :] (+ extra[t, :])   (y float32 [T * top, d])
 // ---------------------------------------------------------------------------------
 __global__ void moe_combine_kernel(float* __restrict__ h, const float* __restrict__ y,
-                                   const float* __restrict__ wgt, const float* __restrict__ extra, int top,
-                                   int d) {
+                                   const float* __restrict__ wgt, const float* __restrict__ extra,
+                                   const float* __restrict__ extra_gate, int ld_gate, int top, int d) {
   const int t = blockIdx.x;
+  const float eg = extra_gate ? 1.0f / (1.0f + expf(-extra_gate[(size_t)t * ld_gate])) : 1.0f;
   for (int i = threadIdx.x; i < d; i += blockDim.x) {
-    float s = extra ? extra[(size_t)t * d + i] : 0.f;
+    float s = extra ? eg * extra[(size_t)t * d + i] : 0.f;
     for (int j = 0; j < top; ++j) s += wgt[(size_t)t * top + j] * y[((size_t)t * top + j) * d + i];
     h[(size_t)t * d + i] += s;
   }
 }
 
-extern "C" int hal_moe_combine(float* h, const float* y, const float* wgt, const float* extra, int top,
-                               int d, int n_tokens, hipStream_t stream) {
+extern "C" int hal_moe_combine(float* h, const float* y, const float* wgt, const float* extra,
+                               const float* extra_gate, int ld_gate, int top, int d, int n_tokens,
+                               hipStream_t stream) {
   HAL_REQUIRE(n_tokens >= 0 && top > 0 && d > 0, "hal_moe_combine: bad sizes");
   if (n_tokens == 0) return 0;
   int threads = (d + 63) / 64 * 64;
   if (threads > 256) threads = 256;
-  hipLaunchKernelGGL(moe_combine_kernel, dim3(n_tokens), dim3(threads), 0, stream, h, y, wgt, extra, top, d);
+  hipLaunchKernelGGL(moe_combine_kernel, dim3(n_tokens), dim3(threads), 0, stream, h, y, wgt, extra, extra_gate, ld_gate, top, d);
   HAL_LAUNCH_CHECK();
   return 0;
 }
@@ -335,17 +337,17 @@ extern "C" int hal_moe_combine(float* h, const float* y, const float* wgt, const
 // ---------------------------------------------------------------------------------
 template <typename T>
 __global__ void clamped_gate_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int F, float limit,
-                                        float alpha) {
+                                        float alpha, float up_shift) {
   const int t = blockIdx.x;
   const int f = blockIdx.y * blockDim.x + threadIdx.x;
   if (f >= F) return;
   const float g = fminf(to_f32(gu[(size_t)t * 2 * F + f]), limit);
   const float u = fminf(fmaxf(to_f32(gu[(size_t)t * 2 * F + F + f]), -limit), limit);
-  out[(size_t)t * F + f] = from_f32<T>(g / (1.0f + __expf(-alpha * g)) * (u + 1.0f));
+  out[(size_t)t * F + f] = from_f32<T>(g / (1.0f + __expf(-alpha * g)) * (u + up_shift));
 }
 
 extern "C" int hal_clamped_gate_mul(const void* gu, void* out, int dtype, int n_tokens, int F,
-                                    float limit, float alpha, hipStream_t stream) {
+                                    float limit, float alpha, float up_shift, hipStream_t stream) {
   HAL_REQUIRE(n_tokens >= 0 && F > 0, "hal_clamped_gate_mul: bad sizes T=%d F=%d", n_tokens, F);
   HAL_REQUIRE(dtype == HAL_F32 || dtype == HAL_BF16, "hal_clamped_gate_mul: dtype %d", dtype);
   HAL_REQUIRE((F + 255) / 256 <= 65535, "hal_clamped_gate_mul: %d columns", F);
@@ -353,10 +355,10 @@ extern "C" int hal_clamped_gate_mul(const void* gu, void* out, int dtype, int n_
   dim3 grid(n_tokens, (F + 255) / 256);
   if (dtype == HAL_F32)
     hipLaunchKernelGGL(clamped_gate_mul_kernel<float>, grid, dim3(256), 0, stream, (const float*)gu,
-                       (float*)out, F, limit, alpha);
+                       (float*)out, F, limit, alpha, up_shift);
   else
     hipLaunchKernelGGL(clamped_gate_mul_kernel<bf16_t>, grid, dim3(256), 0, stream, (const bf16_t*)gu,
-                       (bf16_t*)out, F, limit, alpha);
+                       (bf16_t*)out, F, limit, alpha, up_shift);
   HAL_LAUNCH_CHECK();
   return 0;
 }

@@ -161,7 +161,11 @@ extern "C" int hal_short_conv_carry(const float* u, int ldu, float* state, int t
 //   segment's chunks in order, S <- decay_c S + sums_c, leaving in sums_c the state that
 //   chunk c starts from, and writes the last state to the request's row;
 // MODE 2: a run is a chunk again, walked from the state it starts from, for the outputs.
-// The result is the recurrence's own, token by token; only the order of additions differs. ----
+// The result is the recurrence's own, token by token; only the order of additions differs.
+//
+// `fixed_decay` (or null): float32 [heads], one constant decay a head; then every step size is 1,
+// nothing is added for the token itself, and dt_raw, dt_bias, a_log and d_skip are not read:
+// S <- decay_h S + B x^T, y = S^T C (a linear attention with keys B, queries C, values x). ----
 template <typename T, int NREG, int MODE>
 __global__ void __launch_bounds__(HAL_WAVE)
 ssd_scan_kernel(const T* __restrict__ xbc, int ldx, const float* __restrict__ dt_raw, int ld_dt,
@@ -169,7 +173,7 @@ ssd_scan_kernel(const T* __restrict__ xbc, int ldx, const float* __restrict__ dt
                 int w_dtype, float* __restrict__ state, const int* __restrict__ seg_q_start,
                 const int* __restrict__ seg_q_len, const int* __restrict__ token_slot, float* __restrict__ y,
                 const int* __restrict__ chunks, float* __restrict__ sums, float* __restrict__ decays,
-                int heads, int P, int N, int groups) {
+                int heads, int P, int N, int groups, const float* __restrict__ fixed_decay) {
   __shared__ __align__(16) float bc[2][2 * NREG];
   const int s = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int p = blockIdx.z * HAL_WAVE + lane;
@@ -183,9 +187,11 @@ ssd_scan_kernel(const T* __restrict__ xbc, int ldx, const float* __restrict__ dt
   float S[NREG];
 #pragma unroll
   for (int i = 0; i < NREG; ++i) S[i] = (MODE != 1 && live && i < N) ? st[(size_t)i * P] : 0.f;
-  const float rate = expf(load_as_f32(a_log, w_dtype, h));
-  const float bias = load_as_f32(dt_bias, w_dtype, h);
-  const float skip = load_as_f32(d_skip, w_dtype, h);
+  const bool fixed = fixed_decay != nullptr;
+  const float rate = fixed ? 0.f : expf(load_as_f32(a_log, w_dtype, h));
+  const float bias = fixed ? 0.f : load_as_f32(dt_bias, w_dtype, h);
+  const float skip = fixed ? 0.f : load_as_f32(d_skip, w_dtype, h);
+  const float decay_h = fixed ? fixed_decay[h] : 0.f;
   const size_t b_col = (size_t)inner + (size_t)g * N, c_col = (size_t)inner + (size_t)groups * N + (size_t)g * N;
 
   // a lane brings B[lane], B[lane + 64], .. and the same of C
@@ -211,7 +217,7 @@ ssd_scan_kernel(const T* __restrict__ xbc, int ldx, const float* __restrict__ dt
   };
   ask(t0);
   float x_next = live ? to_f32(xbc[(size_t)t0 * ldx + (size_t)h * P + p]) : 0.f;
-  float dt_next = dt_raw[(size_t)t0 * ld_dt + h];
+  float dt_next = fixed ? 0.f : dt_raw[(size_t)t0 * ld_dt + h];
   float decay_all = 1.f;
   for (int i = 0; i < n; ++i) {
     const int t = t0 + i, buf = i & 1;
@@ -220,13 +226,13 @@ ssd_scan_kernel(const T* __restrict__ xbc, int ldx, const float* __restrict__ dt
     if (i + 1 < n) {
       ask(t + 1);
       x_next = live ? to_f32(xbc[(size_t)(t + 1) * ldx + (size_t)h * P + p]) : 0.f;
-      dt_next = dt_raw[(size_t)(t + 1) * ld_dt + h];
+      if (!fixed) dt_next = dt_raw[(size_t)(t + 1) * ld_dt + h];
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    const float dt = raw > 20.f ? raw : log1pf(expf(raw));
-    const float decay = expf(-rate * dt);
+    const float dt = fixed ? 1.0f : (raw > 20.f ? raw : log1pf(expf(raw)));
+    const float decay = fixed ? decay_h : expf(-rate * dt);
     const float dtx = dt * x;
     if (MODE == 1) {
       decay_all *= decay;
@@ -302,11 +308,13 @@ extern "C" int hal_ssd_scan(const void* xbc, int ldx, int dtype, const float* dt
                             const void* dt_bias, const void* a_log, const void* d_skip, int w_dtype, float* state,
                             const int* seg_q_start, const int* seg_q_len, const int* token_slot, float* y,
                             int n_segs, int heads, int P, int N, int groups, const int* chunks,
-                            const int* seg_chunks, int n_chunks, float* sums, float* decays, hipStream_t stream) {
+                            const int* seg_chunks, int n_chunks, float* sums, float* decays,
+                            const float* fixed_decay, hipStream_t stream) {
   HAL_REQUIRE(n_segs >= 0 && heads > 0 && P > 0 && N > 0 && groups > 0 && heads % groups == 0,
               "hal_ssd_scan: bad sizes segments=%d heads=%d P=%d N=%d groups=%d", n_segs, heads, P, N, groups);
   HAL_REQUIRE(N <= 256, "hal_ssd_scan: a state of %d numbers a channel exceeds 256", N);
-  HAL_REQUIRE(ldx >= heads * P + 2 * groups * N && ld_dt >= heads, "hal_ssd_scan: rows too short");
+  HAL_REQUIRE(ldx >= heads * P + 2 * groups * N && (fixed_decay || ld_dt >= heads), "hal_ssd_scan: rows too short");
+  HAL_REQUIRE(fixed_decay || (dt_raw && dt_bias && a_log && d_skip), "hal_ssd_scan: neither step sizes nor fixed decays");
   HAL_REQUIRE(heads <= 65535 && (P + HAL_WAVE - 1) / HAL_WAVE <= 65535, "hal_ssd_scan: grid limit");
   HAL_REQUIRE(dtype == HAL_F32 || dtype == HAL_BF16, "hal_ssd_scan: dtype %d", dtype);
   const bool cut = chunks != nullptr;
@@ -319,7 +327,7 @@ extern "C" int hal_ssd_scan(const void* xbc, int ldx, int dtype, const float* dt
 #define SCAN_LAUNCH(T_, N_, MODE_, GRID_)                                                                      \
   hipLaunchKernelGGL((ssd_scan_kernel<T_, N_, MODE_>), GRID_, block, 0, stream, (const T_*)xbc, ldx, dt_raw,    \
                      ld_dt, dt_bias, a_log, d_skip, w_dtype, state, seg_q_start, seg_q_len, token_slot, y,     \
-                     chunks, sums, decays, heads, P, N, groups)
+                     chunks, sums, decays, heads, P, N, groups, fixed_decay)
 #define SCAN_STEPS(T_, N_)                                                                                    \
   do {                                                                                                        \
     if (!cut) {                                                                                               \

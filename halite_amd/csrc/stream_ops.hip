@@ -504,6 +504,8 @@ extern "C" int hal_streams_step(float* x, long long copy_stride, int S, const fl
 template <typename T>
 __global__ void head_norm_pack_kernel(const float* __restrict__ q, int ldq, const float* __restrict__ k, int ldk,
                                       const float* __restrict__ v, int ldv, float eps,
+                                      const void* __restrict__ w_q, const void* __restrict__ w_k, int w_dtype,
+                                      bool norm_v, const float* __restrict__ v_other, int ldvo, float v_mix,
                                       const int* __restrict__ positions, T* __restrict__ out, int row_stride,
                                       int n_tokens, int H, int K, int dq, int dv, int D,
                                       const int* __restrict__ token_seg, const int* __restrict__ block_table,
@@ -519,9 +521,15 @@ __global__ void head_norm_pack_kernel(const float* __restrict__ q, int ldq, cons
   const int n = kind == 2 ? dv : dq;
   const float* src = kind == 0 ? q + t * ldq + (size_t)head * dq
                                : (kind == 1 ? k + t * ldk + (size_t)head * dq : v + t * ldv + (size_t)head * dv);
-  float ss = 0.f;
-  for (int i = lane; i < n; i += HAL_WAVE) ss += src[i] * src[i];
-  const float rstd = 1.0f / sqrtf(wave_sum(ss) / (float)n + eps);
+  float rstd = 1.0f;
+  if (kind != 2 || norm_v) {
+    float ss = 0.f;
+    for (int i = lane; i < n; i += HAL_WAVE) ss += src[i] * src[i];
+    rstd = 1.0f / sqrtf(wave_sum(ss) / (float)n + eps);
+  }
+  // (a weight of the head's size, shared by the heads; values: a blend with another layer's)
+  const void* w = kind == 0 ? w_q : (kind == 1 ? w_k : nullptr);
+  const float* other = (kind == 2 && v_other) ? v_other + t * ldvo + (size_t)head * dv : nullptr;
   long long page = -1;
   int off = 0;
   if (k_pages && kind != 0) {
@@ -532,7 +540,10 @@ __global__ void head_norm_pack_kernel(const float* __restrict__ q, int ldq, cons
   }
   T* o = out + t * row_stride + (size_t)hs * D;
   for (int d = lane; d < D; d += HAL_WAVE) {
-    const T x = from_f32<T>(d < n ? src[d] * rstd : 0.f);
+    float f = d < n ? src[d] * rstd : 0.f;
+    if (w && d < n) f *= load_as_f32(w, w_dtype, d);
+    if (other && d < n) f = (1.0f - v_mix) * f + v_mix * other[d];
+    const T x = from_f32<T>(f);
     o[d] = x;
     if (page >= 0) {
       if (kind == 1) k_pages[((size_t)page * K + head) * page_size * D + kv_key_offset(tiled, page_size, D, off, d)] = x;
@@ -542,7 +553,8 @@ __global__ void head_norm_pack_kernel(const float* __restrict__ q, int ldq, cons
 }
 
 extern "C" int hal_head_norm_pack(const float* q, int ldq, const float* k, int ldk, const float* v, int ldv, float eps,
-                                  const int* positions, void* out, int row_stride, int dtype, int n_tokens, int H,
+                                  const void* w_q, const void* w_k, int w_dtype, int norm_v, const float* v_other,
+                                  int ldvo, float v_mix, const int* positions, void* out, int row_stride, int dtype, int n_tokens, int H,
                                   int K, int dq, int dv, int D, const int* token_seg, const int* block_table,
                                   int bt_stride, void* k_pages, void* v_pages, int page_size, int n_pages, int tiled,
                                   hipStream_t stream) {
@@ -553,15 +565,20 @@ extern "C" int hal_head_norm_pack(const float* q, int ldq, const float* k, int l
   HAL_REQUIRE(row_stride >= (H + 2 * K) * D && ldq >= H * dq && ldk >= K * dq && ldv >= K * dv,
               "hal_head_norm_pack: rows too short");
   HAL_REQUIRE(dtype == HAL_F32 || dtype == HAL_BF16, "hal_head_norm_pack: dtype %d", dtype);
+  HAL_REQUIRE((w_q == nullptr) == (w_k == nullptr) && (w_q == nullptr || w_dtype == HAL_F32 || w_dtype == HAL_BF16),
+              "hal_head_norm_pack: weights for both q and k or for neither, float32 or bf16");
+  HAL_REQUIRE(v_other == nullptr || ldvo >= K * dv, "hal_head_norm_pack: rows of the other values too short");
   if (n_tokens == 0) return 0;
   const long long units = (long long)n_tokens * (H + 2 * K);
   const dim3 grid((unsigned)((units + 3) / 4));
   if (dtype == HAL_F32)
-    hipLaunchKernelGGL(head_norm_pack_kernel<float>, grid, dim3(256), 0, stream, q, ldq, k, ldk, v, ldv, eps, positions,
+    hipLaunchKernelGGL(head_norm_pack_kernel<float>, grid, dim3(256), 0, stream, q, ldq, k, ldk, v, ldv, eps, w_q, w_k,
+                       w_dtype, norm_v != 0, v_other, ldvo, v_mix, positions,
                        (float*)out, row_stride, n_tokens, H, K, dq, dv, D, token_seg, block_table, bt_stride,
                        (float*)k_pages, (float*)v_pages, page_size, n_pages, tiled != 0);
   else
-    hipLaunchKernelGGL(head_norm_pack_kernel<bf16_t>, grid, dim3(256), 0, stream, q, ldq, k, ldk, v, ldv, eps, positions,
+    hipLaunchKernelGGL(head_norm_pack_kernel<bf16_t>, grid, dim3(256), 0, stream, q, ldq, k, ldk, v, ldv, eps, w_q, w_k,
+                       w_dtype, norm_v != 0, v_other, ldvo, v_mix, positions,
                        (bf16_t*)out, row_stride, n_tokens, H, K, dq, dv, D, token_seg, block_table, bt_stride,
                        (bf16_t*)k_pages, (bf16_t*)v_pages, page_size, n_pages, tiled != 0);
   HAL_LAUNCH_CHECK();
@@ -593,6 +610,84 @@ extern "C" int hal_head_gate_cols(const void* x, int ldx, int x_head, const floa
   else
     hipLaunchKernelGGL(head_gate_cols_kernel<bf16_t>, dim3(n_tokens), dim3(256), 0, stream, (const bf16_t*)x, ldx, x_head,
                        g, ldg, (bf16_t*)y, n, H);
+  HAL_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---- a[t, c] += bias[c]: the bias of a projection whose float32 result something reads before
+// anything else could add it (a convolution over time, whose inputs before the first token are
+// zeros and not the bias) ------------------------------------------------------------------
+__global__ void bias_rows_kernel(float* __restrict__ a, int lda, const void* __restrict__ bias, int b_dtype, int n_cols) {
+  const size_t t = blockIdx.x;
+  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < n_cols; c += gridDim.y * blockDim.x)
+    a[t * lda + c] += load_as_f32(bias, b_dtype, c);
+}
+
+extern "C" int hal_bias_rows(float* a, int lda, const void* bias, int b_dtype, int n_rows, int n_cols, hipStream_t stream) {
+  HAL_REQUIRE(n_rows >= 0 && n_cols > 0 && lda >= n_cols, "hal_bias_rows: bad sizes rows=%d cols=%d", n_rows, n_cols);
+  HAL_REQUIRE(b_dtype == HAL_F32 || b_dtype == HAL_BF16, "hal_bias_rows: dtype %d", b_dtype);
+  if (n_rows == 0) return 0;
+  const int by = n_cols >= 4096 ? 4 : 1;
+  hipLaunchKernelGGL(bias_rows_kernel, dim3(n_rows, by), dim3(256), 0, stream, a, lda, bias, b_dtype, n_cols);
+  HAL_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---- out[t, c] = silu(a[t, c]) for the first n_cols columns of float32 rows --------------------
+template <typename T>
+__global__ void silu_rows_kernel(const float* __restrict__ a, int lda, T* __restrict__ out, int n_cols) {
+  const size_t t = blockIdx.x;
+  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < n_cols; c += gridDim.y * blockDim.x) {
+    const float z = a[t * lda + c];
+    out[t * n_cols + c] = from_f32<T>(z / (1.0f + expf(-z)));
+  }
+}
+
+extern "C" int hal_silu_rows(const float* a, int lda, void* out, int dtype, int n_rows, int n_cols, hipStream_t stream) {
+  HAL_REQUIRE(n_rows >= 0 && n_cols > 0 && lda >= n_cols, "hal_silu_rows: bad sizes rows=%d cols=%d", n_rows, n_cols);
+  HAL_REQUIRE(dtype == HAL_F32 || dtype == HAL_BF16, "hal_silu_rows: dtype %d", dtype);
+  if (n_rows == 0) return 0;
+  const dim3 grid(n_rows, n_cols >= 4096 ? 4 : 1);
+  if (dtype == HAL_F32)
+    hipLaunchKernelGGL(silu_rows_kernel<float>, grid, dim3(256), 0, stream, a, lda, (float*)out, n_cols);
+  else
+    hipLaunchKernelGGL(silu_rows_kernel<bf16_t>, grid, dim3(256), 0, stream, a, lda, (bf16_t*)out, n_cols);
+  HAL_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---- out[t, j] = gelu_tanh(g[t, j]) * table[tokens[t]][col0 + j]: a small projection of the
+// stream gates the token's own row of a table (a column range of it) ----------------------------
+template <typename T>
+__global__ void token_gate_kernel(const float* __restrict__ g, int ldg, const void* __restrict__ table, int t_dtype,
+                                  int ld_table, int col0, const int* __restrict__ tokens, int vocab,
+                                  T* __restrict__ out, int dim) {
+  const size_t t = blockIdx.x;
+  const int tok = tokens[t];
+  const bool ok = tok >= 0 && tok < vocab;
+  for (int j = threadIdx.x; j < dim; j += blockDim.x) {
+    const float z = g[t * ldg + j];
+    const float act = 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+    const float e = ok ? load_as_f32(table, t_dtype, (size_t)tok * ld_table + col0 + j) : NAN;
+    out[t * dim + j] = from_f32<T>(act * e);
+  }
+}
+
+extern "C" int hal_token_gate(const float* g, int ldg, const void* table, int t_dtype, int ld_table, int col0,
+                              const int* tokens, int vocab, void* out, int dtype, int n_rows, int dim,
+                              hipStream_t stream) {
+  HAL_REQUIRE(n_rows >= 0 && dim > 0 && ldg >= dim && col0 >= 0 && col0 + dim <= ld_table && vocab > 0,
+              "hal_token_gate: bad sizes rows=%d dim=%d col0=%d table row=%d", n_rows, dim, col0, ld_table);
+  HAL_REQUIRE((dtype == HAL_F32 || dtype == HAL_BF16) && (t_dtype == HAL_F32 || t_dtype == HAL_BF16),
+              "hal_token_gate: dtypes %d, %d", dtype, t_dtype);
+  if (n_rows == 0) return 0;
+  const int threads = dim >= 256 ? 256 : (dim > 64 ? 128 : 64);
+  if (dtype == HAL_F32)
+    hipLaunchKernelGGL(token_gate_kernel<float>, dim3(n_rows), dim3(threads), 0, stream, g, ldg, table, t_dtype,
+                       ld_table, col0, tokens, vocab, (float*)out, dim);
+  else
+    hipLaunchKernelGGL(token_gate_kernel<bf16_t>, dim3(n_rows), dim3(threads), 0, stream, g, ldg, table, t_dtype,
+                       ld_table, col0, tokens, vocab, (bf16_t*)out, dim);
   HAL_LAUNCH_CHECK();
   return 0;
 }

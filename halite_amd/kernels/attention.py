@@ -414,6 +414,8 @@ def attention_mfma(q, q_row_stride, plan_dev, ctx, group, kv, n_heads, scale, wi
         ops._need(bias is not None and bias.is_cuda and bias.is_contiguous() and bias.dtype == torch.float32
                   and bias.dim() == 2 and bias.shape[0] == n_heads and bias.shape == rule.bias.shape,
                   "attention: the bias times log2 e is float32 [heads, distances]")
+    sinks = rule.sink_checked(n_heads, log2=True)
+    ops._dev(sinks)
     rc = lib.hal_attention_mfma_ruled(
         P(q), q_row_stride, P(out), n_heads * head_dim,
         P(items), plan.cap_items, P(big_items), plan.cap_big, P(merges), plan.cap_merges, P(counts),
@@ -421,7 +423,7 @@ def attention_mfma(q, q_row_stride, plan_dev, ctx, group, kv, n_heads, scale, wi
         P(group.block_table), group.block_table.shape[1], P(kv.k), P(kv.v), P(part_o), P(part_ml),
         P(counters), N_COUNTERS, n_heads, n_kv, head_dim, page_size, 1 if getattr(kv, "tiled", False) else 0,
         ctypes.c_float(scale), window, rule.chunk, P(bias), 0 if bias is None else bias.shape[1],
-        rule.weights_code(), plan.max_parts, ops._stream(),
+        rule.weights_code(), ctypes.c_float(rule.softcap), P(sinks), plan.max_parts, ops._stream(),
     )
     ops._check(lib, rc)
     return out

@@ -32,7 +32,10 @@ class ScoreRule:
     score of the key ``n`` tokens back at ``[head, min(n, distances - 1)]``.  ``sink``: the
     softmax has one more term of score 0 that carries no value.  ``sigmoid``: no softmax: a
     visible key's weight is the sigmoid of its score (scaled, with the bias), and the weights
-    are not normalised over the keys."""
+    are not normalised over the keys.  ``softcap`` > 0: the scaled score ``s`` becomes
+    ``softcap * tanh(s / softcap)`` before the bias.  ``sink_values`` (with ``sink``): float32
+    ``[heads]`` on the device, the score of the sink's term of every head instead of 0 (it is
+    neither scaled nor capped)."""
 
     chunk: int = 0
     bias: torch.Tensor | None = None
@@ -40,9 +43,23 @@ class ScoreRule:
     # the same table times log2 e, for the kernel whose exponentials are to the base 2
     bias_log2: torch.Tensor | None = None
     sigmoid: bool = False
+    softcap: float = 0.0
+    sink_values: torch.Tensor | None = None
+    # the same values times log2 e
+    sink_values_log2: torch.Tensor | None = None
 
     def plain(self) -> bool:
-        return self.chunk == 0 and self.bias is None and not self.sink and not self.sigmoid
+        return (self.chunk == 0 and self.bias is None and not self.sink and not self.sigmoid
+                and self.softcap == 0.0)
+
+    def sink_checked(self, n_heads: int, log2: bool) -> torch.Tensor | None:
+        """The sinks' values as a kernel takes them (None: every sink has the score 0)."""
+        if self.sink_values is None:
+            return None
+        t = self.sink_values_log2 if log2 else self.sink_values
+        if not self.sink or t is None or t.dtype != torch.float32 or t.shape != (n_heads,) or not t.is_contiguous():
+            raise KernelError("sink values are float32 [heads] (and their multiples of log2 e), with sink=True")
+        return t
 
     def weights_code(self) -> int:
         """The kernels' number for how a row's weights are made (``HAL_WEIGHTS_*``)."""
@@ -386,6 +403,8 @@ def attention_simple(
         _dev(bias)
         _need(bias.dtype == torch.float32 and bias.dim() == 2 and bias.shape[0] == n_heads and bias.shape[1] > 0,
               "attention: the bias is float32 [heads, distances]")
+    sinks = rule.sink_checked(n_heads, log2=False)
+    _dev(sinks)
     _check(
         lib,
         lib.hal_attention_simple_ruled(
@@ -393,7 +412,7 @@ def attention_simple(
             _ptr(positions), _ptr(token_seg), _ptr(block_table), block_table.shape[1],
             _ptr(k_pages), _ptr(v_pages), _ptr(part), n, n_heads, n_kv, head_dim, page_size, n_pages,
             ctypes.c_float(scale), window, rule.chunk, _ptr(bias), 0 if bias is None else bias.shape[1],
-            rule.weights_code(), max_kv_len, min_q_len, _stream(),
+            rule.weights_code(), ctypes.c_float(rule.softcap), _ptr(sinks), max_kv_len, min_q_len, _stream(),
         ),
     )
     return out
@@ -765,20 +784,23 @@ def scale_(x: torch.Tensor, s: float) -> torch.Tensor:
 def grouped_gemm(
     x: torch.Tensor, w: torch.Tensor, y: torch.Tensor, *, n_rows: int,
     x_group_cols: int = 0, x_col0: int = 0, y_group_cols: int = 0, y_col0: int = 0,
-    w_up: torch.Tensor | None = None, limit: float = 0.0, alpha: float = 0.0,
+    w_up: torch.Tensor | None = None, limit: float = 0.0, alpha: float = 0.0, up_shift: float = 1.0,
     group_offsets: torch.Tensor | None = None, tile_offsets: torch.Tensor | None = None,
     row_src: torch.Tensor | None = None, src_div: int = 1, row_dst: torch.Tensor | None = None,
     gate: torch.Tensor | None = None, add: bool = False, mfma: bool = True, relu_squared: bool = False,
+    gate_per_group: bool = False,
 ) -> torch.Tensor:
     """``y_g = x_g @ w[g].T`` for every group ``g`` of ``w`` ``[G, N, K]`` in one launch
     (float32 accumulation).  Heads: every group has all ``n_rows`` rows; group ``g`` reads
     the ``K`` columns from ``g * x_group_cols + x_col0`` of ``x`` and writes the ``N``
     columns from ``g * y_group_cols + y_col0`` of ``y``; ``gate`` (float32, row-strided)
-    multiplies the result by ``sigmoid(gate[t, g * y_group_cols + n])``.  Experts:
+    multiplies the result by ``sigmoid(gate[t, g * y_group_cols + n])`` (``gate_per_group``: by
+    ``sigmoid(gate[t, g])``, one number a group).  Experts:
     ``group_offsets`` / ``tile_offsets`` (from ``moe_sort``) cut a list of ``n_rows`` rows
     into the groups' slices; row ``i`` reads ``x[row_src[i] // src_div]`` and writes
     ``y[row_dst[i]]`` (``i`` without the arrays); with ``w_up`` the result is the clamped
-    gated activation of the two products; without it and with ``relu_squared`` the square of
+    gated activation of the two products, ``g sigmoid(alpha g) (u + up_shift)`` with ``g`` and
+    ``u`` held to ``limit`` (``inf``: not held); without it and with ``relu_squared`` the square of
     the product's positive part.  ``add``: added into a float32 ``y``."""
     lib = library.core_library()
     _dev(w, w_up, group_offsets, tile_offsets, row_src, row_dst)
@@ -795,7 +817,9 @@ def grouped_gemm(
         _need(x.shape[0] >= n_rows and y.shape[0] >= n_rows, "grouped_gemm: rows")
         _need((g - 1) * x_group_cols + x_col0 + k <= x.shape[1] and (g - 1) * y_group_cols + y_col0 + n <= y.shape[1],
               "grouped_gemm: columns outside the rows")
-        _need(gate is None or (gate.shape[0] >= n_rows and (g - 1) * y_group_cols + n <= gate.shape[1]), "grouped_gemm: gate")
+        _need(gate is None or (gate.shape[0] >= n_rows and
+                               (g <= gate.shape[1] if gate_per_group else (g - 1) * y_group_cols + n <= gate.shape[1])),
+              "grouped_gemm: gate")
     else:
         _need(group_offsets.numel() == g + 1 and tile_offsets is not None and tile_offsets.numel() == g + 1, "grouped_gemm: offsets")
         _need(x_group_cols == 0 and y_group_cols == 0 and x_col0 + k <= x.shape[1] and y_col0 + n <= y.shape[1], "grouped_gemm: columns")
@@ -808,7 +832,8 @@ def grouped_gemm(
         _ptr(x), x.stride(0), x_group_cols, x_col0, _ptr(w), _ptr(w_up), ctypes.c_longlong(n * k), k,
         dtype_code(x.dtype), _ptr(y), y.stride(0), y_group_cols, y_col0, dtype_code(y.dtype), 1 if add else 0,
         n_rows, n, k, g, _ptr(group_offsets), _ptr(tile_offsets), _ptr(row_src), src_div, _ptr(row_dst),
-        _ptr(gate), 0 if gate is None else gate.stride(0), ctypes.c_float(limit), ctypes.c_float(alpha),
+        _ptr(gate), 0 if gate is None else gate.stride(0), 1 if gate_per_group else 0, ctypes.c_float(limit),
+        ctypes.c_float(up_shift), ctypes.c_float(alpha),
         1 if relu_squared else 0, 1 if mfma else 0, _stream()))
     return y
 
@@ -818,12 +843,12 @@ def moe_route(z: torch.Tensor, top: int, softmax: bool = False, normalize: bool 
     ``[T, top]`` int32 and weights ``[T, top]`` float32 (sigmoid scores, or the softmax over
     the experts; divided by their sum + ``norm_eps`` if ``normalize``)."""
     lib = library.core_library()
-    _dev(z)
-    _need(z.dtype == torch.float32 and z.dim() == 2, "moe_route: float32 logits [T, E]")
+    _need(z.is_cuda and z.dtype == torch.float32 and z.dim() == 2 and z.stride(1) == 1,
+          "moe_route: float32 logits [T, E] (a row-strided view is allowed)")
     t, e = z.shape
     idx = torch.empty((t, top), dtype=torch.int32, device=z.device)
     wgt = torch.empty((t, top), dtype=torch.float32, device=z.device)
-    _check(lib, lib.hal_moe_route(_ptr(z), e, top, 1 if softmax else 0, 1 if normalize else 0,
+    _check(lib, lib.hal_moe_route(_ptr(z), z.stride(0), e, top, 1 if softmax else 0, 1 if normalize else 0,
                                   ctypes.c_float(norm_eps), _ptr(idx), _ptr(wgt), t, _stream()))
     return idx, wgt
 
@@ -843,19 +868,26 @@ def moe_sort(idx: torch.Tensor, n_experts: int):
     return offsets, tile_offsets, order
 
 
-def moe_combine(h: torch.Tensor, y: torch.Tensor, wgt: torch.Tensor, extra: torch.Tensor | None = None) -> None:
-    """``h[t] += sum_j wgt[t, j] * y[t * top + j] (+ extra[t])`` (all float32)."""
+def moe_combine(h: torch.Tensor, y: torch.Tensor, wgt: torch.Tensor, extra: torch.Tensor | None = None,
+                extra_gate: torch.Tensor | None = None) -> None:
+    """``h[t] += sum_j wgt[t, j] * y[t * top + j] (+ extra[t])`` (all float32); with
+    ``extra_gate`` (float32 ``[T, 1]``, a row-strided view is allowed) ``extra[t]`` is
+    multiplied by ``sigmoid(extra_gate[t])``."""
     lib = library.core_library()
     _dev(h, y, wgt, extra)
     t, top = wgt.shape
     _need(extra is None or (extra.dtype == torch.float32 and extra.shape == h.shape), "moe_combine: extra like h")
     _need(h.dtype == y.dtype == wgt.dtype == torch.float32 and h.shape[0] == t and y.shape == (t * top, h.shape[1]),
           "moe_combine: float32 h [T, d], y [T * top, d], weights [T, top]")
-    _check(lib, lib.hal_moe_combine(_ptr(h), _ptr(y), _ptr(wgt), _ptr(extra), top, h.shape[1], t, _stream()))
+    if extra_gate is not None:
+        _need(extra is not None and extra_gate.is_cuda and extra_gate.dtype == torch.float32
+              and extra_gate.shape == (t, 1), "moe_combine: a float32 gate [T, 1] for the extra rows")
+    _check(lib, lib.hal_moe_combine(_ptr(h), _ptr(y), _ptr(wgt), _ptr(extra), _ptr(extra_gate),
+                                    0 if extra_gate is None else extra_gate.stride(0), top, h.shape[1], t, _stream()))
 
 
-def clamped_gate_mul(gate_up: torch.Tensor, limit: float, alpha: float) -> torch.Tensor:
-    """``g * sigmoid(alpha * g) * (u + 1)`` with ``g = min(gate, limit)`` and
+def clamped_gate_mul(gate_up: torch.Tensor, limit: float, alpha: float, up_shift: float = 1.0) -> torch.Tensor:
+    """``g * sigmoid(alpha * g) * (u + up_shift)`` with ``g = min(gate, limit)`` and
     ``u = clamp(up, -limit, limit)`` of rows ``[gate | up]``."""
     lib = library.core_library()
     _dev(gate_up)
@@ -863,7 +895,7 @@ def clamped_gate_mul(gate_up: torch.Tensor, limit: float, alpha: float) -> torch
     _need(two_f % 2 == 0, "clamped_gate_mul: odd row length")
     out = torch.empty((n, two_f // 2), dtype=gate_up.dtype, device=gate_up.device)
     _check(lib, lib.hal_clamped_gate_mul(_ptr(gate_up), _ptr(out), dtype_code(gate_up.dtype), n, two_f // 2,
-                                         ctypes.c_float(limit), ctypes.c_float(alpha), _stream()))
+                                         ctypes.c_float(limit), ctypes.c_float(alpha), ctypes.c_float(up_shift), _stream()))
     return out
 
 
@@ -1041,24 +1073,31 @@ def short_conv_carry(u: torch.Tensor, state: torch.Tensor, seg_q_start: torch.Te
 def ssd_scan(xbc: torch.Tensor, dt_raw: torch.Tensor, dt_bias: torch.Tensor, a_log: torch.Tensor,
              d_skip: torch.Tensor, state: torch.Tensor, seg_q_start: torch.Tensor, seg_q_len: torch.Tensor,
              token_slot: torch.Tensor, groups: int, chunks: torch.Tensor | None = None,
-             seg_chunks: torch.Tensor | None = None) -> torch.Tensor:
+             seg_chunks: torch.Tensor | None = None, fixed_decay: torch.Tensor | None = None) -> torch.Tensor:
     """The state-space recurrence over every request's tokens of the step.  ``xbc``
     ``[T, heads * P + 2 * groups * N]``: x, then B and C; ``dt_raw`` float32 ``[T, heads]``
     (a row-strided view is allowed); ``state`` float32 ``[slots, heads, N, P]``, read and
     left as the step's last state.  Returns float32 ``[T, heads * P]``.  ``chunks`` int32
     ``[n, 4]`` (first token, tokens, segment, 0) and ``seg_chunks`` ``[segments, 2]`` (first
     chunk, chunks): the segments cut into chunks that are walked side by side (what long
-    prompts need to fill the chip); without them a wave walks a whole segment."""
+    prompts need to fill the chip); without them a wave walks a whole segment.
+    ``fixed_decay`` float32 ``[heads]``: one constant decay a head, every step size 1 and nothing
+    added for the token itself (``dt_raw``, ``dt_bias``, ``a_log`` and ``d_skip`` are None):
+    ``S <- decay S + B x^T``, ``y = S^T C``."""
     lib = library.core_library()
-    _dev(xbc, dt_bias, a_log, d_skip, state, seg_q_start, seg_q_len, token_slot)
+    _dev(xbc, dt_bias, a_log, d_skip, state, seg_q_start, seg_q_len, token_slot, fixed_decay)
     _, heads, n_state, p = state.shape
     n = xbc.shape[0]
     _need(state.dtype == torch.float32 and xbc.dim() == 2 and xbc.shape[1] == heads * p + 2 * groups * n_state,
           "ssd_scan: rows of x, B and C")
-    _need(dt_raw.is_cuda and dt_raw.dtype == torch.float32 and dt_raw.shape == (n, heads) and dt_raw.stride(1) == 1,
-          "ssd_scan: float32 step sizes [T, heads]")
-    _need(dt_bias.numel() == heads and a_log.numel() == heads and d_skip.numel() == heads
-          and dt_bias.dtype == a_log.dtype == d_skip.dtype, "ssd_scan: one bias, rate and skip a head, of one type")
+    if fixed_decay is not None:
+        _need(fixed_decay.dtype == torch.float32 and fixed_decay.shape == (heads,) and dt_raw is None and dt_bias is None
+              and a_log is None and d_skip is None, "ssd_scan: fixed decays are float32 [heads] and come alone")
+    else:
+        _need(dt_raw.is_cuda and dt_raw.dtype == torch.float32 and dt_raw.shape == (n, heads) and dt_raw.stride(1) == 1,
+              "ssd_scan: float32 step sizes [T, heads]")
+        _need(dt_bias.numel() == heads and a_log.numel() == heads and d_skip.numel() == heads
+              and dt_bias.dtype == a_log.dtype == d_skip.dtype, "ssd_scan: one bias, rate and skip a head, of one type")
     y = torch.empty((n, heads * p), dtype=torch.float32, device=xbc.device)
     sums = decays = None
     n_chunks = 0
@@ -1071,10 +1110,10 @@ def ssd_scan(xbc: torch.Tensor, dt_raw: torch.Tensor, dt_bias: torch.Tensor, a_l
         sums = torch.empty((n_chunks, heads, n_state, p), dtype=torch.float32, device=xbc.device)
         decays = torch.empty((n_chunks, heads), dtype=torch.float32, device=xbc.device)
     _check(lib, lib.hal_ssd_scan(
-        _ptr(xbc), xbc.shape[1], dtype_code(xbc.dtype), _ptr(dt_raw), dt_raw.stride(0), _ptr(dt_bias), _ptr(a_log),
-        _ptr(d_skip), dtype_code(a_log.dtype), _ptr(state), _ptr(seg_q_start), _ptr(seg_q_len), _ptr(token_slot),
+        _ptr(xbc), xbc.shape[1], dtype_code(xbc.dtype), _ptr(dt_raw), 0 if dt_raw is None else dt_raw.stride(0),
+        _ptr(dt_bias), _ptr(a_log), _ptr(d_skip), F32 if a_log is None else dtype_code(a_log.dtype), _ptr(state), _ptr(seg_q_start), _ptr(seg_q_len), _ptr(token_slot),
         _ptr(y), seg_q_start.numel(), heads, p, n_state, groups, _ptr(chunks), _ptr(seg_chunks), n_chunks,
-        _ptr(sums), _ptr(decays), _stream()))
+        _ptr(sums), _ptr(decays), _ptr(fixed_decay), _stream()))
     return y
 
 
@@ -1189,12 +1228,23 @@ def head_norm_pack(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, eps: float
                    qk_dim: int, v_dim: int, head_dim: int, out_dtype: torch.dtype,
                    positions: torch.Tensor | None = None, token_seg: torch.Tensor | None = None,
                    block_table: torch.Tensor | None = None, k_pages: torch.Tensor | None = None,
-                   v_pages: torch.Tensor | None = None, page_size: int = 0, tiled: bool = False) -> torch.Tensor:
+                   v_pages: torch.Tensor | None = None, page_size: int = 0, tiled: bool = False,
+                   w_q: torch.Tensor | None = None, w_k: torch.Tensor | None = None, norm_v: bool = True,
+                   v_other: torch.Tensor | None = None, v_mix: float = 0.0) -> torch.Tensor:
     """From float32 projections (row-strided views allowed): every head of ``q``, ``k`` and
-    ``v`` divided by its own root mean square (no weight); the packed rows ``[q heads | k heads
-    | v heads]`` of ``head_dim`` entries a head (zero beyond ``qk_dim`` / ``v_dim``) come back.
+    (with ``norm_v``) ``v`` divided by its own root mean square; the packed rows ``[q heads | k
+    heads | v heads]`` of ``head_dim`` entries a head (zero beyond ``qk_dim`` / ``v_dim``) come
+    back.  ``w_q`` / ``w_k`` ``[qk_dim]``: a weight that multiplies every normed head of q / k.
+    ``v_other`` (float32 rows like ``v``): the values become ``(1 - v_mix) v + v_mix v_other``.
     With ``k_pages`` and ``v_pages`` keys and values are appended to the pages as well."""
     lib = library.core_library()
+    _dev(w_q, w_k)
+    _need((w_q is None) == (w_k is None) and (w_q is None or (w_q.shape == (qk_dim,) and w_k.shape == (qk_dim,)
+                                                             and w_q.dtype == w_k.dtype)),
+          "head_norm_pack: weights [qk_dim] of one type for q and k, or none")
+    if v_other is not None:
+        _rows_f32(v_other, n_kv_heads * v_dim, "head_norm_pack v_other")
+        _need(v_other.shape[0] == q.shape[0], "head_norm_pack: one row of other values a token")
     n = q.shape[0]
     _rows_f32(q, n_heads * qk_dim, "head_norm_pack q"), _rows_f32(k, n_kv_heads * qk_dim, "head_norm_pack k")
     _rows_f32(v, n_kv_heads * v_dim, "head_norm_pack v")
@@ -1211,7 +1261,9 @@ def head_norm_pack(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, eps: float
         _need(positions is not None and positions.numel() == n and token_seg is not None and token_seg.numel() == n
               and block_table is not None and block_table.dim() == 2, "head_norm_pack: the step's arrays")
     _check(lib, lib.hal_head_norm_pack(
-        _ptr(q), q.stride(0), _ptr(k), k.stride(0), _ptr(v), v.stride(0), ctypes.c_float(eps), _ptr(positions),
+        _ptr(q), q.stride(0), _ptr(k), k.stride(0), _ptr(v), v.stride(0), ctypes.c_float(eps),
+        _ptr(w_q), _ptr(w_k), dtype_code(w_q.dtype) if w_q is not None else F32, 1 if norm_v else 0,
+        _ptr(v_other), 0 if v_other is None else v_other.stride(0), ctypes.c_float(v_mix), _ptr(positions),
         _ptr(out), out.shape[1], dtype_code(out_dtype), n, n_heads, n_kv_heads, qk_dim, v_dim, head_dim,
         _ptr(token_seg), _ptr(block_table), 0 if block_table is None else block_table.shape[1],
         _ptr(k_pages), _ptr(v_pages), page_size, n_pages, 1 if tiled else 0, _stream()))
@@ -1231,3 +1283,39 @@ def head_gate_cols(x: torch.Tensor, x_head: int, gate: torch.Tensor, n: int, n_h
     _check(lib, lib.hal_head_gate_cols(_ptr(x), x.shape[1], x_head, _ptr(gate), gate.stride(0), _ptr(y), n, n_heads,
                                        dtype_code(x.dtype), x.shape[0], _stream()))
     return y
+
+
+# -- small passes over float32 rows of projections ----------------------------------------------
+
+
+def bias_rows_(a: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
+    """``a[t, c] += bias[c]`` in place on float32 rows (a row-strided view is allowed)."""
+    lib = library.core_library()
+    _dev(bias)
+    _rows_f32(a, bias.numel(), "bias_rows_")
+    _check(lib, lib.hal_bias_rows(_ptr(a), a.stride(0), _ptr(bias), dtype_code(bias.dtype), a.shape[0], a.shape[1], _stream()))
+    return a
+
+
+def silu_rows(a: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """``silu(a)`` of float32 rows (a row-strided view is allowed), rounded to ``out_dtype``."""
+    lib = library.core_library()
+    _rows_f32(a, a.shape[1], "silu_rows")
+    out = torch.empty(a.shape, dtype=out_dtype, device=a.device)
+    _check(lib, lib.hal_silu_rows(_ptr(a), a.stride(0), _ptr(out), dtype_code(out_dtype), a.shape[0], a.shape[1], _stream()))
+    return out
+
+
+def token_gate(g: torch.Tensor, table: torch.Tensor, col0: int, tokens: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """``gelu_tanh(g[t, j]) * table[tokens[t], col0 + j]`` for float32 rows ``g`` ``[T, dim]``
+    and a table ``[vocab, columns]``; a token outside the table gives a NaN row."""
+    lib = library.core_library()
+    _dev(table, tokens)
+    _i32(tokens, "tokens")
+    n, dim = g.shape
+    _rows_f32(g, dim, "token_gate")
+    _need(table.dim() == 2 and 0 <= col0 and col0 + dim <= table.shape[1] and tokens.numel() == n, "token_gate: sizes")
+    out = torch.empty((n, dim), dtype=out_dtype, device=g.device)
+    _check(lib, lib.hal_token_gate(_ptr(g), g.stride(0), _ptr(table), dtype_code(table.dtype), table.shape[1], col0,
+                                   _ptr(tokens), table.shape[0], _ptr(out), dtype_code(out_dtype), n, dim, _stream()))
+    return out

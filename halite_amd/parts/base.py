@@ -104,6 +104,8 @@ class BuildContext:
     positions: dict[str, "Part"] = field(default_factory=dict)
     # keep a second copy of every bf16 matrix in the small-batch kernel's tiled order
     tiled_weights: bool = False
+    # the model's embedding, once it is built (parts of the layers may read tables it owns)
+    embedding: "Embedding | None" = None
 
 
 @dataclass

@@ -110,15 +110,19 @@ class PostNormBlock(Arrangement):
     for the part that reads them next."""
 
     graph_safe = True
-    roles = {"mixer": MIXERS, "mixer_norm": NORMS, "ff": FEED_FORWARDS, "ff_norm": NORMS}
-    optional = ("ff", "ff_norm")
+    roles = {"mixer": MIXERS, "mixer_norm": NORMS, "ff": FEED_FORWARDS, "ff_norm": NORMS,
+             "side": FEED_FORWARDS, "side_norm": NORMS}
+    optional = ("ff", "ff_norm", "side", "side_norm")
 
     def __init__(self, parts):
         super().__init__(parts)
         self.mixer_norm, self.ff_norm, self.ff = parts["mixer_norm"], parts.get("ff_norm"), parts.get("ff")
-        if (self.ff is None) != (self.ff_norm is None):
-            raise ValueError("a post-norm block has a feed-forward and its norm, or neither")
-        for norm in (self.mixer_norm, self.ff_norm):
+        # a third part of the feed-forward kind that closes the layer the same way:
+        # h = h + norm_c(side(h))
+        self.side, self.side_norm = parts.get("side"), parts.get("side_norm")
+        if (self.ff is None) != (self.ff_norm is None) or (self.side is None) != (self.side_norm is None):
+            raise ValueError("a post-norm block has a feed-forward (a side part) and its norm, or neither")
+        for norm in (self.mixer_norm, self.ff_norm, self.side_norm):
             if norm is not None and not isinstance(norm, RMSNorm):
                 raise ValueError(f"a post-norm block norms with RMSNorm; {type(norm).__name__} is another")
 
@@ -135,12 +139,12 @@ class PostNormBlock(Arrangement):
         else:
             x = ops.cast_rows(h, dtype)
         norm = self.mixer_norm
-        last = self.ff is None
+        weight_of = lambda nm: getattr(nm, "multiplier", nm.weight)  # noqa: E731
         # a sum of two mixers is made by the kernel that norms it
         terms = self.mixer.forward_terms(x, ctx, run) if hasattr(self.mixer, "forward_terms") else None
         if terms is not None and len(terms) == 2:
             (a, s1), (b, s2) = terms
-            x = ops.post_norm_add(h, a, norm.weight, norm.p.eps, cast_to=dtype, scale=s1, second=b, second_scale=s2)
+            x = ops.post_norm_add(h, a, weight_of(norm), norm.p.eps, cast_to=dtype, scale=s1, second=b, second_scale=s2)
         else:
             a = self.mixer.forward(x, ctx, run) if terms is None else None
             if terms is not None:  # any other number of members: added up one by one
@@ -149,12 +153,14 @@ class PostNormBlock(Arrangement):
                     ops.scaled_sum_(a, 1.0, b, s)
             if a.dtype != torch.float32:
                 a = a.float()
-            x = ops.post_norm_add(h, a, norm.weight, norm.p.eps, cast_to=dtype)
-        if not last:
-            b = self.ff.forward(x, ctx)
+            x = ops.post_norm_add(h, a, weight_of(norm), norm.p.eps, cast_to=dtype)
+        for part, part_norm in ((self.ff, self.ff_norm), (self.side, self.side_norm)):
+            if part is None:
+                continue
+            b = part.forward(x, ctx)
             if b.dtype != torch.float32:
                 b = b.float()
-            x = ops.post_norm_add(h, b, self.ff_norm.weight, self.ff_norm.p.eps, cast_to=dtype)
+            x = ops.post_norm_add(h, b, weight_of(part_norm), part_norm.p.eps, cast_to=dtype)
         if dtype != torch.float32:
             ctx.rounded_rows = (run.index, x)
         return None

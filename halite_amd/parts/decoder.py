@@ -39,8 +39,9 @@ class Decoder:
     def __init__(self, spec: ModelSpec, dtype: torch.dtype, device: torch.device | str,
                  tiled_weights: bool = False):
         # the kinds of parts register themselves when their modules are imported
-        from . import (attention, block, connection, embedding, feedforward, general_delta, latent_attention,  # noqa: F401
-                       mixer_sum, moe, norm, normed_attention, rope, sigmoid_attention, state_space)
+        from . import (attention, block, capped_attention, connection, decay_attention, embedding, feedforward,  # noqa: F401
+                       general_delta, latent_attention, mixer_sum, moe, norm, normed_attention, rope,
+                       sigmoid_attention, state_space, token_gated)
 
         self.spec = spec
         self.dtype = dtype
@@ -52,6 +53,7 @@ class Decoder:
         self.build = build
         self.positions = build.positions
         self.embedding = EMBEDDINGS.build(spec.embedding, build)
+        build.embedding = self.embedding
         self.layers = {}
         for name, lspec in spec.layers.items():
             if lspec.arrangement not in ARRANGEMENTS:

@@ -15,6 +15,12 @@ class EmbeddingParams(BaseModel):
     size: StrictInt = Field(gt=0)
     scale: float = 1.0
     """Every row is multiplied by this on its way into the stream (in float32)."""
+    norm_eps: float | None = Field(default=None, gt=0)
+    """With a value: a tensor ``norm.weight`` of the rows' size, and every row enters the
+    stream as ``x / sqrt(mean(x^2) + norm_eps) * weight`` (float32)."""
+    side_size: StrictInt | None = Field(default=None, gt=0)
+    """With a value: a second table ``side.weight`` ``[vocab_size, side_size]`` of which parts of
+    the layers read column ranges by token (``BuildContext.embedding.side_weight``)."""
 
 
 @EMBEDDINGS.register("embedding")
@@ -26,10 +32,22 @@ class TokenEmbedding(Embedding):
     graph_safe = True
 
     def param_decls(self):
-        return {"weight": ParamDecl((self.p.vocab_size, self.p.size))}
+        decls = {"weight": ParamDecl((self.p.vocab_size, self.p.size))}
+        if self.p.norm_eps is not None:
+            decls["norm.weight"] = ParamDecl((self.p.size,), init="ones")
+        if self.p.side_size is not None:
+            decls["side.weight"] = ParamDecl((self.p.vocab_size, self.p.side_size))
+        return decls
 
     def forward(self, tokens, out=None):
-        return ops.embedding(tokens, self.weight, out=out, scale=self.p.scale)
+        if self.p.norm_eps is None:
+            return ops.embedding(tokens, self.weight, out=out, scale=self.p.scale)
+        x = ops.rmsnorm_exact(ops.embedding(tokens, self.weight, scale=self.p.scale), self.norm_weight, self.p.norm_eps,
+                              torch.float32)
+        if out is None:
+            return x
+        out.copy_(x)
+        return out
 
 
 class LinearHeadParams(BaseModel):

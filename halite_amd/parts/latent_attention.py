@@ -41,14 +41,22 @@ class LatentAttentionParams(BaseModel):
     window: StrictInt | None = Field(default=None, gt=0)
     output_gate: StrictBool = False
     """The concatenated heads are multiplied by ``sigmoid(W_g x)`` before the output projection."""
+    gate_per_head: StrictBool = False
+    """With ``output_gate``: ``W_g`` has one row a head, and a head's result is multiplied by
+    one number."""
+    learned_sink: StrictBool = False
+    """Every head's softmax has one more term in its denominator, ``exp(sink[head])`` with a
+    tensor ``sink`` ``[n_heads]``: it has no key and no value and is not scaled."""
+    float32_result: StrictBool = False
+    """True: without a stream to add into, the output projection's float32 sums come back unrounded."""
 
 
 @MIXERS.register("latent_attention")
 class LatentAttention(Mixer):
     """``c_q = norm(W_dq x)``, ``q = W_uq c_q`` (per head ``[nope_dim | rope_dim]``);
     ``[c' | r] = W_dkv x``, ``c = norm(c')``; rotation of ``q``'s rotated part and of ``r``;
-    causal softmax attention inside ``window`` as described above; optional output gate;
-    output projection."""
+    causal softmax attention inside ``window`` as described above (optionally with a learned
+    sink a head); optional output gate; output projection."""
 
     Params = LatentAttentionParams
     graph_safe = True
@@ -64,8 +72,8 @@ class LatentAttention(Mixer):
             if p.position not in build.positions:
                 raise ValueError(f"latent attention names position encoding {p.position!r}, which the model does not define")
             self.position = build.positions[p.position]
-            if not isinstance(self.position, RotaryPositionEncoding) or self.position.interleaved:
-                raise ValueError(f"latent attention rotates pairs (j, j + n/2); position encoding {p.position!r} does not")
+            if not isinstance(self.position, RotaryPositionEncoding):
+                raise ValueError(f"position encoding {p.position!r} is not a RotaryPositionEncoding")
             if self.position.rotary_dim > p.rope_dim:
                 raise ValueError("the position encoding rotates more elements than the rotated part has")
         elif p.rope_dim:
@@ -85,7 +93,9 @@ class LatentAttention(Mixer):
             "out.weight": ParamDecl((d, h * p.v_dim)),
         }
         if p.output_gate:
-            decls["gate.weight"] = ParamDecl((h * p.v_dim, d))
+            decls["gate.weight"] = ParamDecl((h if p.gate_per_head else h * p.v_dim, d))
+        if p.learned_sink:
+            decls["sink"] = ParamDecl((h,))
         return decls
 
     def allocate(self, dtypes):
@@ -116,6 +126,11 @@ class LatentAttention(Mixer):
         # the latent's space
         self.w_ukt = self.w_uk.view(h, p.nope_dim, p.kv_rank).transpose(1, 2).contiguous()
         self.w_uv3 = self.w_uv.view(h, p.v_dim, p.kv_rank)
+        self.rule = None
+        if p.learned_sink:
+            sinks = self.w_sink.float().contiguous()
+            self.rule = ops.ScoreRule(sink=True, sink_values=sinks,
+                                      sink_values_log2=(sinks.double() * 1.4426950408889634).float().contiguous())
         self.t_down = self.t_uq = self.t_out = None
         if self.build.tiled_weights and self.w_down.is_cuda:
             tile = lambda w: ops.tile_weight(w) if w.dtype == torch.bfloat16 and w.shape[1] % 8 == 0 else None  # noqa: E731
@@ -157,15 +172,16 @@ class LatentAttention(Mixer):
             cos = sin = ctx.empty_f32
             rot = 0
         ops.rope_append(
-            packed, ctx.positions, cos, sin, h, 1 if run.appends else 0, D, rot, False,
+            packed, ctx.positions, cos, sin, h, 1 if run.appends else 0, D, rot,
+            self.position.interleaved if self.position is not None else False,
             token_seg=ctx.token_seg, block_table=group.block_table,
             k_pages=kv.k, v_pages=kv.v, page_size=group.page_size, tiled=kv.tiled,
         )
-        latent = ctx.attention(packed, packed.shape[1], kv, group, h, p.scale, p.window or 0)
+        latent = ctx.attention(packed, packed.shape[1], kv, group, h, p.scale, p.window or 0, rule=self.rule)
         heads = torch.empty((n, h * p.v_dim), dtype=x.dtype, device=x.device)
         ops.grouped_gemm(latent, self.w_uv3, heads, n_rows=n, x_group_cols=D, x_col0=p.rope_dim, y_group_cols=p.v_dim,
-                         gate=a[:, gate_col0:] if p.output_gate else None)
+                         gate=a[:, gate_col0:] if p.output_gate else None, gate_per_group=p.gate_per_head)
         if add_to is not None:
             ops.linear_add(add_to, heads, self.w_out, tiled=self.t_out)
             return None
-        return ops.linear(heads, self.w_out, tiled=self.t_out)
+        return ops.linear(heads, self.w_out, out_dtype=torch.float32 if p.float32_result else None, tiled=self.t_out)

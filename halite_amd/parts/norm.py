@@ -20,10 +20,17 @@ class RMSNormParams(BaseModel):
     """The stored weight is the multiplier's distance from this: the norm multiplies by
     ``weight_offset + weight`` (float32; only in the unrounded order)."""
 
+    layer_scale: StrictBool = False
+    """True: a second tensor ``scale`` of the norm's size multiplies the result element by
+    element (a learned scale on what a part adds to the stream); the two are multiplied once,
+    in float32, when the weights are loaded (only in the unrounded order)."""
+
     @model_validator(mode="after")
     def _check(self):
         if self.weight_offset != 0.0 and self.round_before_weight:
             raise ValueError("a weight stored as a distance is added up in float32: round_before_weight must be false")
+        if self.layer_scale and (self.round_before_weight or self.weight_offset != 0.0):
+            raise ValueError("a layer scale comes with the unrounded order and a plain weight")
         return self
 
 
@@ -38,9 +45,21 @@ class RMSNorm(Norm):
     graph_safe = True
 
     def param_decls(self):
-        return {"weight": ParamDecl((self.p.size,), init="ones")}
+        decls = {"weight": ParamDecl((self.p.size,), init="ones")}
+        if self.p.layer_scale:
+            decls["scale"] = ParamDecl((self.p.size,), init="ones")
+        return decls
+
+    def finalize(self):
+        # what multiplies the normalised rows: the weight, or weight * scale in float32 (exact
+        # for two 16-bit factors)
+        self.multiplier = self.weight.float() * self.scale.float() if self.p.layer_scale else self.weight
 
     def forward(self, h, delta=None, rows=None):
+        if self.p.layer_scale:
+            if delta is not None:
+                ops.residual_add(h, delta)
+            return ops.rmsnorm_exact(h, self.multiplier, self.p.eps, self.build.dtype, rows=rows)
         if not self.p.round_before_weight:
             if delta is not None:
                 ops.residual_add(h, delta)

@@ -43,13 +43,35 @@ class LinearFrequencyScaling(BaseModel):
     factor: float = Field(gt=0)
 
 
+class RampFrequencyScaling(BaseModel):
+    """Frequencies blended with themselves divided by ``factor`` along a ramp over the pair
+    index ``i``: with ``at(turns) = rotary_dim * ln(original_context_len / (2 pi turns)) /
+    (2 ln theta)`` (the index whose wavelength fits ``turns`` times into the original
+    context), ``lo = max(floor(at(fast_turns)), 0)`` and ``hi = min(ceil(at(slow_turns)),
+    rotary_dim - 1)``, the pair ``i`` gets ``f_i / factor * r + f_i * (1 - r)`` with
+    ``r = clamp((i - lo) / max(hi - lo, 0.001), 0, 1)``: fast pairs are kept, slow ones
+    stretched.  An architecture's description translates its own keys into these."""
+
+    model_config = ConfigDict(extra="forbid")
+
+    kind: Literal["ramp"]
+    factor: float = Field(gt=0)
+    original_context_len: StrictInt = Field(gt=0)
+    fast_turns: float = Field(gt=0)
+    slow_turns: float = Field(gt=0)
+
+
 class RopeParams(BaseModel):
     head_dim: StrictInt = Field(gt=0)
     rotary_dim: StrictInt = Field(gt=0)
     theta: float = Field(gt=0)
     interleaved: StrictBool = False
     max_positions: StrictInt = Field(gt=0)
-    scaling: BandedFrequencyScaling | LinearFrequencyScaling | None = Field(default=None, discriminator="kind")
+    scaling: BandedFrequencyScaling | LinearFrequencyScaling | RampFrequencyScaling | None = Field(
+        default=None, discriminator="kind")
+    magnitude: float = Field(default=1.0, gt=0)
+    """Cosine and sine are multiplied by this (a rotated query and key then carry it twice in
+    their product)."""
     angles: Literal["float32", "float64"] = "float32"
     """The arithmetic in which frequencies and angles are computed before cosine and sine
     are rounded to the float32 table (float32: as the reference computes them)."""
@@ -75,6 +97,15 @@ def rope_inverse_frequencies(p: RopeParams) -> torch.Tensor:
         return inv_freq
     if isinstance(s, LinearFrequencyScaling):
         return inv_freq / s.factor
+    if isinstance(s, RampFrequencyScaling):
+        def at(turns: float) -> float:
+            return p.rotary_dim * math.log(s.original_context_len / (2 * math.pi * turns)) / (2 * math.log(p.theta))
+
+        lo = max(math.floor(at(s.fast_turns)), 0)
+        hi = min(math.ceil(at(s.slow_turns)), p.rotary_dim - 1)
+        index = torch.arange(p.rotary_dim // 2, dtype=real, device="cpu")
+        ramp = ((index - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+        return inv_freq / s.factor * ramp + inv_freq * (1 - ramp)
     long_wavelen = s.original_context_len / s.low_freq_factor
     short_wavelen = s.original_context_len / s.high_freq_factor
     wavelen = 2 * math.pi / inv_freq
@@ -118,6 +149,6 @@ class Rope(RotaryPositionEncoding):
             n = max(n, min(self.p.max_positions, 4096))
             t = torch.arange(n, dtype=self.inv_freq.dtype, device="cpu")
             angles = torch.outer(t, self.inv_freq)
-            self._cos = angles.cos().float().to(self.build.device).contiguous()
-            self._sin = angles.sin().float().to(self.build.device).contiguous()
+            self._cos = (angles.cos() * self.p.magnitude).float().to(self.build.device).contiguous()
+            self._sin = (angles.sin() * self.p.magnitude).float().to(self.build.device).contiguous()
         return self._cos, self._sin

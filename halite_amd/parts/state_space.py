@@ -24,6 +24,34 @@ from .base import MIXERS, Mixer, ParamDecl, StateNeed
 SCAN_CHUNK = 64
 
 
+def plan_scan_chunks(ctx) -> None:
+    """Long segments are cut into chunks that are walked side by side; the cut depends on
+    the segments' token counts alone and is shared by every layer of the step that scans
+    (``scan_arrays`` gives a layer the arrays, if the step has them)."""
+    lens = ctx.seg_q_len_host
+    if ctx.static is not None or len(lens) == 0 or int(lens.max()) < 2 * SCAN_CHUNK:
+        return
+    per_seg = -(-lens.astype(np.int64) // SCAN_CHUNK)
+    first = np.concatenate(([0], np.cumsum(per_seg)[:-1]))
+
+    def chunks():
+        seg = np.repeat(np.arange(len(lens)), per_seg)
+        k = np.arange(int(per_seg.sum())) - first[seg]
+        t0 = ctx.seg_q_start_host[seg] + k * SCAN_CHUNK
+        n = np.minimum(SCAN_CHUNK, lens[seg] - k * SCAN_CHUNK)
+        return np.stack((t0, n, seg, np.zeros_like(seg)), axis=1)
+
+    ctx.add_array(f"scan_chunks_{SCAN_CHUNK}", chunks)
+    ctx.add_array(f"scan_seg_chunks_{SCAN_CHUNK}", lambda: np.stack((first, per_seg), axis=1))
+
+
+def scan_arrays(ctx) -> dict:
+    """``chunks`` and ``seg_chunks`` for ``ops.ssd_scan`` (None where the step is not cut)."""
+    cut = ctx.has_array(f"scan_chunks_{SCAN_CHUNK}")
+    return dict(chunks=ctx.array(f"scan_chunks_{SCAN_CHUNK}") if cut else None,
+                seg_chunks=ctx.array(f"scan_seg_chunks_{SCAN_CHUNK}") if cut else None)
+
+
 class StateSpaceParams(BaseModel):
     hidden_size: StrictInt = Field(gt=0)
     n_heads: StrictInt = Field(gt=0)
@@ -91,23 +119,7 @@ class StateSpace(Mixer):
         return need
 
     def prepare(self, ctx, run):
-        # Long segments are cut into chunks that are walked side by side; the cut depends on
-        # the segments' token counts alone and is shared by every layer of the step.
-        lens = ctx.seg_q_len_host
-        if ctx.static is not None or len(lens) == 0 or int(lens.max()) < 2 * SCAN_CHUNK:
-            return
-        per_seg = -(-lens.astype(np.int64) // SCAN_CHUNK)
-        first = np.concatenate(([0], np.cumsum(per_seg)[:-1]))
-
-        def chunks():
-            seg = np.repeat(np.arange(len(lens)), per_seg)
-            k = np.arange(int(per_seg.sum())) - first[seg]
-            t0 = ctx.seg_q_start_host[seg] + k * SCAN_CHUNK
-            n = np.minimum(SCAN_CHUNK, lens[seg] - k * SCAN_CHUNK)
-            return np.stack((t0, n, seg, np.zeros_like(seg)), axis=1)
-
-        ctx.add_array(f"scan_chunks_{SCAN_CHUNK}", chunks)
-        ctx.add_array(f"scan_seg_chunks_{SCAN_CHUNK}", lambda: np.stack((first, per_seg), axis=1))
+        plan_scan_chunks(ctx)
 
     def forward(self, x, ctx, run):
         p = self.p
@@ -118,10 +130,7 @@ class StateSpace(Mixer):
         dt_raw = a[:, inner + self.conv_channels :]
         conv_state = run.state["conv"] if p.conv_taps > 1 else a.new_zeros((1, 0, self.conv_channels))
         xbc = ops.short_conv_through(u, self.conv_weight, self.conv_bias, conv_state, ctx, x.dtype, silu=True)
-        cut = ctx.has_array(f"scan_chunks_{SCAN_CHUNK}")
         y = ops.ssd_scan(xbc, dt_raw, self.dt_bias, self.A_log, self.D, run.state["state"], ctx.seg_q_start,
-                         ctx.seg_q_len, ctx.token_slot, p.groups,
-                         chunks=ctx.array(f"scan_chunks_{SCAN_CHUNK}") if cut else None,
-                         seg_chunks=ctx.array(f"scan_seg_chunks_{SCAN_CHUNK}") if cut else None)
+                         ctx.seg_q_len, ctx.token_slot, p.groups, **scan_arrays(ctx))
         gated = ops.gated_part_norm(y, z, self.norm_weight, p.eps, p.norm_parts, x.dtype)
         return ops.linear(gated, self.out_weight, out_dtype=torch.float32, tiled=self.t_out)
