@@ -101,7 +101,7 @@ class Families:
     ELEMENTWISE = ("rmsnorm", "silu_mul", "rope_append", "embedding", "residual_add", "rmsnorm_exact", "latent_prep",
                    "head_cols", "scale_", "moe_route", "moe_sort", "moe_combine", "clamped_gate_mul", "cast_rows",
                    "post_norm_add", "relu_squared", "scaled_sum_", "qk_norm_pack", "gated_part_norm", "head_norm_gate",
-                   "streams_step", "head_norm_pack", "head_gate_cols")
+                   "streams_step", "head_norm_pack", "head_gate_cols", "bias_rows_", "silu_rows", "token_gate")
     RECURRENT = ("short_conv", "short_conv_carry", "ssd_scan", "delta_rule")
 
     def __init__(self):
@@ -484,6 +484,72 @@ def vepitar_work(s, n_layers, tokens, batch=0, kv_tokens=0, elt=2, window=0) -> 
             "recurrent": 2.0 * batch * n_delta * 2 * state * 4 / elt}
 
 
+# Layers of the Diporax design at the same two sizes: to every four layers two of the capped
+# attention (biased projections, convolutions of four taps, a weighted norm per head, half of
+# every head rotated, values blended with the first layer's), one latent attention with a sink and
+# one linear attention with constant decays whose state is as large as the delta rule's; every
+# layer with sixteen gated experts of which a token uses four, a shared expert behind its gate,
+# and the token input.  Beside it Vepitar layers of the same width and heads: the closest
+# design that the engine serves (attentions with convolutions and a gate per head beside
+# recurrences with a float32 state per request, and routed experts).
+DIPORAX_SIZES = {
+    "2048-wide": dict(VEPITAR_SIZES["2048-wide"], rot_dim=64, q_rank=768, kv_rank=192, decay_heads=32, decay_dim=64,
+                      gated_ff=1024, shared_ff=1024, side=128),
+    "4096-wide": dict(VEPITAR_SIZES["4096-wide"], rot_dim=64, q_rank=1536, kv_rank=192, decay_heads=64, decay_dim=64,
+                      gated_ff=2048, shared_ff=2048, side=256),
+}
+
+
+def diporax_layer_kinds(n_layers):
+    return [("attention", "attention", "latent_attention", "lightning")[i % 4] for i in range(n_layers)]
+
+
+def diporax_config(s, n_layers, window):
+    rot = dict(base=500000.0, dims=64, scaling=dict(factor=4.0, original=2048, fast=32.0, slow=1.0))
+    attention = dict(heads=s["heads"], kv_heads=s["kv_heads"], dim=s["dim"], vdim=s["dim"], scale=s["dim"] ** -0.5,
+                     conv=s["conv"], rot=rot, softcap=30.0, v_mix=True, bias=True)
+    latent = dict(heads=s["heads"], dim=s["dim"], rot_dim=s["rot_dim"], vdim=s["dim"], q_rank=s["q_rank"],
+                  kv_rank=s["kv_rank"], scale=(s["dim"] + s["rot_dim"]) ** -0.5, rot=rot)
+    lightning = dict(heads=s["decay_heads"], dim=s["decay_dim"], vdim=s["decay_dim"],
+                     decay=[1.0 - 2.0 ** -(5 + 8 * h / s["decay_heads"]) for h in range(s["decay_heads"])])
+    mixers = {"attention": attention, "latent_attention": latent, "lightning": lightning}
+    moe = dict(kind="moe", router=dict(experts=s["experts"], top=s["top"]), expert=dict(ff=s["gated_ff"]),
+               shared=dict(ff=s["shared_ff"]))
+    return dict(architecture="Diporax", vocab=COMPARISON_VOCAB, width=s["width"], norm=dict(eps=1e-6),
+                token_side=dict(dim=s["side"]), max_positions=8192,
+                layers=[dict(type=kind, mixer=mixers[kind], mlp=moe) for kind in diporax_layer_kinds(n_layers)])
+
+
+def diporax_work(s, n_layers, tokens, batch=0, kv_tokens=0, elt=2) -> dict:
+    """As ``vepitar_work``; the family ``recurrent`` is the convolutions and the linear attention
+    (four float32 operations per token and entry of a head's state: decay and write, read), whose
+    decode step reads and writes every request's state."""
+    d, h, kv, D = s["width"], s["heads"], s["kv_heads"], s["dim"]
+    kinds = diporax_layer_kinds(n_layers)
+    n_att, n_lat, n_dec = kinds.count("attention"), kinds.count("latent_attention"), kinds.count("lightning")
+    DL = -(-(s["rot_dim"] + s["kv_rank"]) // 16) * 16
+    inner = s["decay_heads"] * s["decay_dim"]
+    att = d * ((h + 2 * kv) * D + h) + h * D * d
+    lat = d * (s["q_rank"] + s["kv_rank"] + s["rot_dim"] + h) + s["q_rank"] * h * (D + s["rot_dim"]) + h * D * d
+    dec = d * 4 * inner + inner * d
+    every = d * (s["experts"] + 1) + s["shared_ff"] * d + 2 * d * s["side"]  # router, shared down, token input
+    linear = n_att * att + n_lat * lat + n_dec * dec + n_layers * every
+    heads = n_lat * (h * D * s["kv_rank"] + h * s["kv_rank"] * D)
+    shared_in = 2 * d * s["shared_ff"]
+    expert = 3 * d * s["gated_ff"]
+    state = s["decay_heads"] * s["decay_dim"] * s["decay_dim"]
+    if batch == 0:
+        return {"gemm": 2.0 * tokens * linear + 2.0 * COMPARISON_VOCAB * d,
+                "grouped": 2.0 * tokens * (heads + n_layers * (shared_in + s["top"] * expert)),
+                "attention": 2.0 * tokens * tokens * h * (D * n_att + DL * n_lat),
+                "recurrent": tokens * (n_dec * 4.0 * state + n_att * 2.0 * s["conv"] * (h + 2 * kv) * D)}
+    used = min(s["experts"], batch * s["top"])
+    return {"gemm": 2.0 * (linear + COMPARISON_VOCAB * d),
+            "grouped": 2.0 * (heads + n_layers * (shared_in + used * expert)),
+            "attention": 2.0 * kv_tokens * (2 * kv * D * n_att + 2 * DL * n_lat),
+            "recurrent": 2.0 * batch * n_dec * 2 * state * 4 / elt}
+
+
 DESIGNS = {
     "kavuvik": dict(label="Kavuvik", sizes=lambda: KAVUVIK_SIZES, config=lambda s, n, w: kavuvik_config(s, n, w),
                     llama=lambda s, n: closest_llama_config(s, n),
@@ -495,11 +561,15 @@ DESIGNS = {
                     beside=dict(key="zabunex", label="Zabunex", config=lambda s, n: zabunex_config(s, n, 0),
                                 work=lambda s, n, t, b, kv, elt: zabunex_work(s, n, t, b, kv, elt)),
                     work=lambda s, n, t, b, kv, elt, w=0: vepitar_work(s, n, t, b, kv, elt, w)),
+    "diporax": dict(label="Diporax", sizes=lambda: DIPORAX_SIZES, config=lambda s, n, w: diporax_config(s, n, w),
+                    beside=dict(key="vepitar", label="Vepitar", config=lambda s, n: vepitar_config(s, n, 0),
+                                work=lambda s, n, t, b, kv, elt: vepitar_work(s, n, t, b, kv, elt, 0)),
+                    work=lambda s, n, t, b, kv, elt: diporax_work(s, n, t, b, kv, elt)),
 }
 
 
 def design_comparison(args) -> dict:
-    """``--workload kavuvik`` / ``zabunex``: prefill and decode throughput of the design's
+    """``--workload kavuvik`` / ``zabunex`` / ``vepitar`` / ``diporax``: prefill and decode throughput of the design's
     layers at two sizes beside the closest Llama layers, with each family of kernels against
     its roofline (the products and the attention of a prompt against the bf16 matrix peak, a
     recurrence against the float32 vector peak, those of a decode step against the memory's
@@ -654,7 +724,7 @@ def main() -> int:
                          "by default (scheduling_steps_ahead); 0: read every step's tokens before the next is put together")
     ap.add_argument("--sampling", default="greedy", choices=["greedy", "temperature", "top_p", "top_k", "all"],
                     help="how the decode steps sample (the contract's line is greedy)")
-    ap.add_argument("--workload", default="decode8b", choices=["decode8b", "mixed3b", "llama70b", "kavuvik", "zabunex", "vepitar"],
+    ap.add_argument("--workload", default="decode8b", choices=["decode8b", "mixed3b", "llama70b", "kavuvik", "zabunex", "vepitar", "diporax"],
                     help="decode8b: the headline line; mixed3b and llama70b run requests through the scheduler; "
                          "kavuvik, zabunex: prefill and decode of that design's layers at two sizes beside the closest Llama layers; "
                          "vepitar: the same beside Zabunex layers of equal size")

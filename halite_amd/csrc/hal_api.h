@@ -225,17 +225,21 @@ int hal_qk_norm_pack(const float* q, int ldq, const float* k, int ldk, const flo
 // y[t, c] = act(bias[c] + sum_j w[c, j] * u[t - taps + 1 + j, c]) over the tokens of each
 // request, the inputs before a step's first token taken from state [slots][taps - 1][C]
 // (float32; zero for a new request).  act: 0 none, 1 silu.  w [C, taps], bias [C] or null.
-int hal_short_conv(const float* u, int ldu, const void* w, const void* bias, int w_dtype, int taps,
+// in_bias (or null; here and in the two entry points below): [C], added to every input u[t, c]
+// where it is read (not to the zeros before a request's first token)
+int hal_short_conv(const float* u, int ldu, const void* w, const void* bias, int w_dtype,
+                   const void* in_bias, int ib_dtype, int taps,
                    const float* state, const int* token_seg, const int* seg_q_start,
                    const int* token_slot, void* y, int ldy, int y_dtype, int act, int n_tokens,
                    int C, hipStream_t stream);
 // Both in one kernel for a step in which every request brings one token (token t belongs to
 // slot token_slot[t], no two tokens to the same): y as above, and the state moved one on.
 int hal_short_conv_step(const float* u, int ldu, const void* w, const void* bias, int w_dtype,
-                        int taps, float* state, const int* token_slot, void* y, int ldy,
+                        const void* in_bias, int ib_dtype, int taps, float* state, const int* token_slot, void* y, int ldy,
                         int y_dtype, int act, int n_tokens, int C, hipStream_t stream);
 // The state after the step: the last taps - 1 of (the state, then the step's inputs).
-int hal_short_conv_carry(const float* u, int ldu, float* state, int taps, const int* seg_q_start,
+int hal_short_conv_carry(const float* u, int ldu, const void* in_bias, int ib_dtype, float* state, int taps,
+                         const int* seg_q_start,
                          const int* seg_q_len, const int* token_slot, int n_segs, int C,
                          hipStream_t stream);
 // xbc [T, ldx]: x (heads * P), then B and C (groups * N each).  state [slots][heads][N][P].
@@ -244,12 +248,13 @@ int hal_short_conv_carry(const float* u, int ldu, float* state, int taps, const 
 // floats) and decays (n_chunks * heads floats): the segments cut into chunks that are walked
 // side by side, or all null: a wave walks a whole segment.  fixed_decay (or null): float32
 // [heads], one constant decay a head with step sizes of 1 and no D: S <- decay S + B x^T.
+// in_silu: x, B and C are SiLU of what xbc holds.
 int hal_ssd_scan(const void* xbc, int ldx, int dtype, const float* dt_raw, int ld_dt,
                  const void* dt_bias, const void* a_log, const void* d_skip, int w_dtype,
                  float* state, const int* seg_q_start, const int* seg_q_len, const int* token_slot,
                  float* y, int n_segs, int heads, int P, int N, int groups, const int* chunks,
                  const int* seg_chunks, int n_chunks, float* sums, float* decays,
-                 const float* fixed_decay, hipStream_t stream);
+                 const float* fixed_decay, int in_silu, hipStream_t stream);
 // out = (y * silu(z)) / rms over each of `parts` equal parts of the row * w
 int hal_gated_part_norm(const float* y, const float* z, int ldz, const void* w, int w_dtype,
                         float eps, void* out, int dtype, int n_tokens, int inner, int parts,

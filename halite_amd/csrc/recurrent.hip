@@ -6,6 +6,8 @@
 // segment where its tokens start and how many there are.
 //
 //   y[t, c] = act(bias[c] + sum_j w[c, j] * u[t - taps + 1 + j, c])   (u = 0 before a request's start)
+//   (with `in_bias`, u[t, c] stands for u[t, c] + in_bias[c] wherever a token's input is read: the
+//   bias of the projection that made u, which the zeros before a request's start do not get)
 //   S_t = exp(-exp(A_log) * dt_t) S_(t-1) + dt_t * B_t x_t^T,  y_t = S_t^T C_t + D x_t,
 //   dt_t = softplus(dt_raw_t + dt_bias)
 //
@@ -22,7 +24,8 @@ __device__ __forceinline__ float silu_f32(float x) { return x / (1.0f + expf(-x)
 // state [slots][taps - 1][C]: the last taps - 1 inputs of the request before this step
 template <typename TY>
 __global__ void short_conv_kernel(const float* __restrict__ u, int ldu, const void* __restrict__ w,
-                                  const void* __restrict__ bias, int w_dtype, int taps,
+                                  const void* __restrict__ bias, int w_dtype, const void* __restrict__ in_bias,
+                                  int ib_dtype, int taps,
                                   const float* __restrict__ state, const int* __restrict__ token_seg,
                                   const int* __restrict__ seg_q_start, const int* __restrict__ token_slot,
                                   TY* __restrict__ y, int ldy, int act, int n_tokens, int C) {
@@ -32,9 +35,10 @@ __global__ void short_conv_kernel(const float* __restrict__ u, int ldu, const vo
   const int i = t - seg_q_start[token_seg[t]];  // the token's place in its segment
   const float* st = state + (size_t)token_slot[t] * (taps - 1) * C;
   float acc = bias ? load_as_f32(bias, w_dtype, c) : 0.f;
+  const float ib = in_bias ? load_as_f32(in_bias, ib_dtype, c) : 0.f;
   for (int j = 0; j < taps; ++j) {
     const int back = taps - 1 - j;  // how many tokens before t
-    const float x = back <= i ? u[(size_t)(t - back) * ldu + c] : st[(size_t)(taps - 1 - (back - i)) * C + c];
+    const float x = back <= i ? u[(size_t)(t - back) * ldu + c] + ib : st[(size_t)(taps - 1 - (back - i)) * C + c];
     acc = fmaf(load_as_f32(w, w_dtype, (size_t)c * taps + j), x, acc);
   }
   if (act == 1) acc = silu_f32(acc);
@@ -45,14 +49,15 @@ __global__ void short_conv_kernel(const float* __restrict__ u, int ldu, const vo
 // one kernel; a thread owns its (request, channel) and moves the carried inputs one on.
 template <typename TY>
 __global__ void short_conv_step_kernel(const float* __restrict__ u, int ldu, const void* __restrict__ w,
-                                       const void* __restrict__ bias, int w_dtype, int taps,
+                                       const void* __restrict__ bias, int w_dtype, const void* __restrict__ in_bias,
+                                       int ib_dtype, int taps,
                                        float* __restrict__ state, const int* __restrict__ token_slot,
                                        TY* __restrict__ y, int ldy, int act, int C) {
   const int c = blockIdx.y * blockDim.x + threadIdx.x;
   const int t = blockIdx.x;
   if (c >= C) return;
   float* st = state + (size_t)token_slot[t] * (taps - 1) * C + c;
-  const float x = u[(size_t)t * ldu + c];
+  const float x = u[(size_t)t * ldu + c] + (in_bias ? load_as_f32(in_bias, ib_dtype, c) : 0.f);
   float acc = bias ? load_as_f32(bias, w_dtype, c) : 0.f;
   float old[CONV_MAX_TAPS];
 #pragma unroll
@@ -70,7 +75,8 @@ __global__ void short_conv_step_kernel(const float* __restrict__ u, int ldu, con
   y[(size_t)t * ldy + c] = from_f32<TY>(acc);
 }
 
-extern "C" int hal_short_conv_step(const float* u, int ldu, const void* w, const void* bias, int w_dtype, int taps,
+extern "C" int hal_short_conv_step(const float* u, int ldu, const void* w, const void* bias, int w_dtype,
+                                   const void* in_bias, int ib_dtype, int taps,
                                    float* state, const int* token_slot, void* y, int ldy, int y_dtype, int act,
                                    int n_tokens, int C, hipStream_t stream) {
   HAL_REQUIRE(n_tokens >= 0 && C > 0 && taps >= 1 && taps <= CONV_MAX_TAPS && ldu >= C && ldy >= C,
@@ -81,16 +87,17 @@ extern "C" int hal_short_conv_step(const float* u, int ldu, const void* w, const
   if (n_tokens == 0) return 0;
   dim3 grid(n_tokens, (C + 255) / 256);
   if (y_dtype == HAL_F32)
-    hipLaunchKernelGGL(short_conv_step_kernel<float>, grid, dim3(256), 0, stream, u, ldu, w, bias, w_dtype, taps, state,
-                       token_slot, (float*)y, ldy, act, C);
+    hipLaunchKernelGGL(short_conv_step_kernel<float>, grid, dim3(256), 0, stream, u, ldu, w, bias, w_dtype, in_bias, ib_dtype,
+                       taps, state, token_slot, (float*)y, ldy, act, C);
   else
-    hipLaunchKernelGGL(short_conv_step_kernel<bf16_t>, grid, dim3(256), 0, stream, u, ldu, w, bias, w_dtype, taps, state,
-                       token_slot, (bf16_t*)y, ldy, act, C);
+    hipLaunchKernelGGL(short_conv_step_kernel<bf16_t>, grid, dim3(256), 0, stream, u, ldu, w, bias, w_dtype, in_bias, ib_dtype,
+                       taps, state, token_slot, (bf16_t*)y, ldy, act, C);
   HAL_LAUNCH_CHECK();
   return 0;
 }
 
-extern "C" int hal_short_conv(const float* u, int ldu, const void* w, const void* bias, int w_dtype, int taps,
+extern "C" int hal_short_conv(const float* u, int ldu, const void* w, const void* bias, int w_dtype,
+                              const void* in_bias, int ib_dtype, int taps,
                               const float* state, const int* token_seg, const int* seg_q_start,
                               const int* token_slot, void* y, int ldy, int y_dtype, int act, int n_tokens, int C,
                               hipStream_t stream) {
@@ -102,17 +109,18 @@ extern "C" int hal_short_conv(const float* u, int ldu, const void* w, const void
   if (n_tokens == 0) return 0;
   dim3 grid(n_tokens, (C + 255) / 256);
   if (y_dtype == HAL_F32)
-    hipLaunchKernelGGL(short_conv_kernel<float>, grid, dim3(256), 0, stream, u, ldu, w, bias, w_dtype, taps, state,
-                       token_seg, seg_q_start, token_slot, (float*)y, ldy, act, n_tokens, C);
+    hipLaunchKernelGGL(short_conv_kernel<float>, grid, dim3(256), 0, stream, u, ldu, w, bias, w_dtype, in_bias, ib_dtype, taps,
+                       state, token_seg, seg_q_start, token_slot, (float*)y, ldy, act, n_tokens, C);
   else
-    hipLaunchKernelGGL(short_conv_kernel<bf16_t>, grid, dim3(256), 0, stream, u, ldu, w, bias, w_dtype, taps, state,
-                       token_seg, seg_q_start, token_slot, (bf16_t*)y, ldy, act, n_tokens, C);
+    hipLaunchKernelGGL(short_conv_kernel<bf16_t>, grid, dim3(256), 0, stream, u, ldu, w, bias, w_dtype, in_bias, ib_dtype, taps,
+                       state, token_seg, seg_q_start, token_slot, (bf16_t*)y, ldy, act, n_tokens, C);
   HAL_LAUNCH_CHECK();
   return 0;
 }
 
 // ---- what the convolution carries to the next step: a thread a (segment, channel) ---------
-__global__ void short_conv_carry_kernel(const float* __restrict__ u, int ldu, float* __restrict__ state, int taps,
+__global__ void short_conv_carry_kernel(const float* __restrict__ u, int ldu, const void* __restrict__ in_bias,
+                                        int ib_dtype, float* __restrict__ state, int taps,
                                         const int* __restrict__ seg_q_start, const int* __restrict__ seg_q_len,
                                         const int* __restrict__ token_slot, int C) {
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
@@ -121,13 +129,14 @@ __global__ void short_conv_carry_kernel(const float* __restrict__ u, int ldu, fl
   const int t0 = seg_q_start[s], n = seg_q_len[s];
   if (n <= 0) return;
   float* st = state + (size_t)token_slot[t0] * (taps - 1) * C;
+  const float ib = in_bias ? load_as_f32(in_bias, ib_dtype, c) : 0.f;
   float keep[CONV_MAX_TAPS];
   // the last taps - 1 of (what was carried, then the step's inputs)
 #pragma unroll
   for (int i = 0; i < CONV_MAX_TAPS - 1; ++i) {
     if (i < taps - 1) {
       const int at = n + i;  // place in the joined row, whose first taps - 1 are the old ones
-      keep[i] = at < taps - 1 ? st[(size_t)at * C + c] : u[(size_t)(t0 + at - (taps - 1)) * ldu + c];
+      keep[i] = at < taps - 1 ? st[(size_t)at * C + c] : u[(size_t)(t0 + at - (taps - 1)) * ldu + c] + ib;
     }
   }
 #pragma unroll
@@ -135,14 +144,15 @@ __global__ void short_conv_carry_kernel(const float* __restrict__ u, int ldu, fl
     if (i < taps - 1) st[(size_t)i * C + c] = keep[i];
 }
 
-extern "C" int hal_short_conv_carry(const float* u, int ldu, float* state, int taps, const int* seg_q_start,
+extern "C" int hal_short_conv_carry(const float* u, int ldu, const void* in_bias, int ib_dtype, float* state, int taps,
+                                    const int* seg_q_start,
                                     const int* seg_q_len, const int* token_slot, int n_segs, int C,
                                     hipStream_t stream) {
   HAL_REQUIRE(n_segs >= 0 && n_segs <= 65535 && C > 0 && taps >= 1 && taps <= CONV_MAX_TAPS && ldu >= C,
               "hal_short_conv_carry: bad sizes segments=%d C=%d taps=%d", n_segs, C, taps);
   if (n_segs == 0 || taps == 1) return 0;
-  hipLaunchKernelGGL(short_conv_carry_kernel, dim3((C + 255) / 256, n_segs), dim3(256), 0, stream, u, ldu, state,
-                     taps, seg_q_start, seg_q_len, token_slot, C);
+  hipLaunchKernelGGL(short_conv_carry_kernel, dim3((C + 255) / 256, n_segs), dim3(256), 0, stream, u, ldu, in_bias,
+                     ib_dtype, state, taps, seg_q_start, seg_q_len, token_slot, C);
   HAL_LAUNCH_CHECK();
   return 0;
 }
@@ -165,7 +175,9 @@ extern "C" int hal_short_conv_carry(const float* u, int ldu, float* state, int t
 //
 // `fixed_decay` (or null): float32 [heads], one constant decay a head; then every step size is 1,
 // nothing is added for the token itself, and dt_raw, dt_bias, a_log and d_skip are not read:
-// S <- decay_h S + B x^T, y = S^T C (a linear attention with keys B, queries C, values x). ----
+// S <- decay_h S + B x^T, y = S^T C (a linear attention with keys B, queries C, values x).
+// `in_silu`: x, B and C are what SiLU makes of the numbers in `xbc` (the activation of the
+// projections that made them, applied as they are read). ----
 template <typename T, int NREG, int MODE>
 __global__ void __launch_bounds__(HAL_WAVE)
 ssd_scan_kernel(const T* __restrict__ xbc, int ldx, const float* __restrict__ dt_raw, int ld_dt,
@@ -173,7 +185,7 @@ ssd_scan_kernel(const T* __restrict__ xbc, int ldx, const float* __restrict__ dt
                 int w_dtype, float* __restrict__ state, const int* __restrict__ seg_q_start,
                 const int* __restrict__ seg_q_len, const int* __restrict__ token_slot, float* __restrict__ y,
                 const int* __restrict__ chunks, float* __restrict__ sums, float* __restrict__ decays,
-                int heads, int P, int N, int groups, const float* __restrict__ fixed_decay) {
+                int heads, int P, int N, int groups, const float* __restrict__ fixed_decay, bool in_silu) {
   __shared__ __align__(16) float bc[2][2 * NREG];
   const int s = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int p = blockIdx.z * HAL_WAVE + lane;
@@ -197,12 +209,16 @@ ssd_scan_kernel(const T* __restrict__ xbc, int ldx, const float* __restrict__ dt
   // a lane brings B[lane], B[lane + 64], .. and the same of C
   constexpr int PER = (NREG + HAL_WAVE - 1) / HAL_WAVE;
   float nb[PER], nc[PER];
+  auto in = [&](size_t at) {
+    const float v = to_f32(xbc[at]);
+    return in_silu ? silu_f32(v) : v;
+  };
   auto ask = [&](int t) {
 #pragma unroll
     for (int u = 0; u < PER; ++u) {
       const int i = lane + u * HAL_WAVE;
-      nb[u] = i < N ? to_f32(xbc[(size_t)t * ldx + b_col + i]) : 0.f;
-      if (MODE != 1) nc[u] = i < N ? to_f32(xbc[(size_t)t * ldx + c_col + i]) : 0.f;
+      nb[u] = i < N ? in((size_t)t * ldx + b_col + i) : 0.f;
+      if (MODE != 1) nc[u] = i < N ? in((size_t)t * ldx + c_col + i) : 0.f;
     }
   };
   auto put = [&](int buf) {
@@ -216,7 +232,7 @@ ssd_scan_kernel(const T* __restrict__ xbc, int ldx, const float* __restrict__ dt
     }
   };
   ask(t0);
-  float x_next = live ? to_f32(xbc[(size_t)t0 * ldx + (size_t)h * P + p]) : 0.f;
+  float x_next = live ? in((size_t)t0 * ldx + (size_t)h * P + p) : 0.f;
   float dt_next = fixed ? 0.f : dt_raw[(size_t)t0 * ld_dt + h];
   float decay_all = 1.f;
   for (int i = 0; i < n; ++i) {
@@ -225,7 +241,7 @@ ssd_scan_kernel(const T* __restrict__ xbc, int ldx, const float* __restrict__ dt
     const float x = x_next, raw = dt_next + bias;
     if (i + 1 < n) {
       ask(t + 1);
-      x_next = live ? to_f32(xbc[(size_t)(t + 1) * ldx + (size_t)h * P + p]) : 0.f;
+      x_next = live ? in((size_t)(t + 1) * ldx + (size_t)h * P + p) : 0.f;
       if (!fixed) dt_next = dt_raw[(size_t)(t + 1) * ld_dt + h];
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -309,7 +325,7 @@ extern "C" int hal_ssd_scan(const void* xbc, int ldx, int dtype, const float* dt
                             const int* seg_q_start, const int* seg_q_len, const int* token_slot, float* y,
                             int n_segs, int heads, int P, int N, int groups, const int* chunks,
                             const int* seg_chunks, int n_chunks, float* sums, float* decays,
-                            const float* fixed_decay, hipStream_t stream) {
+                            const float* fixed_decay, int in_silu, hipStream_t stream) {
   HAL_REQUIRE(n_segs >= 0 && heads > 0 && P > 0 && N > 0 && groups > 0 && heads % groups == 0,
               "hal_ssd_scan: bad sizes segments=%d heads=%d P=%d N=%d groups=%d", n_segs, heads, P, N, groups);
   HAL_REQUIRE(N <= 256, "hal_ssd_scan: a state of %d numbers a channel exceeds 256", N);
@@ -327,7 +343,7 @@ extern "C" int hal_ssd_scan(const void* xbc, int ldx, int dtype, const float* dt
 #define SCAN_LAUNCH(T_, N_, MODE_, GRID_)                                                                      \
   hipLaunchKernelGGL((ssd_scan_kernel<T_, N_, MODE_>), GRID_, block, 0, stream, (const T_*)xbc, ldx, dt_raw,    \
                      ld_dt, dt_bias, a_log, d_skip, w_dtype, state, seg_q_start, seg_q_len, token_slot, y,     \
-                     chunks, sums, decays, heads, P, N, groups, fixed_decay)
+                     chunks, sums, decays, heads, P, N, groups, fixed_decay, in_silu != 0)
 #define SCAN_STEPS(T_, N_)                                                                                    \
   do {                                                                                                        \
     if (!cut) {                                                                                               \

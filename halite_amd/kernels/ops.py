@@ -1006,15 +1006,18 @@ def qk_norm_pack(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor | None, w_q: 
 
 def short_conv(u: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, state: torch.Tensor,
                token_seg: torch.Tensor, seg_q_start: torch.Tensor, token_slot: torch.Tensor,
-               out_dtype: torch.dtype, silu: bool = False) -> torch.Tensor:
+               out_dtype: torch.dtype, silu: bool = False, in_bias: torch.Tensor | None = None) -> torch.Tensor:
     """The causal convolution over time ``y[t, c] = act(bias[c] + sum_j weight[c, j] *
     u[t - taps + 1 + j, c])`` on the step's flat batch: ``u`` float32 ``[T, C]`` (a
     row-strided view is allowed), ``state`` float32 ``[slots, taps - 1, C]`` the inputs of
-    every request before this step (zeros for a new one; not changed here)."""
+    every request before this step (zeros for a new one; not changed here).  ``in_bias``
+    ``[C]``: added to every input of the step where it is read (the bias of the projection that
+    made ``u``; the state rows hold inputs with it, the zeros before a request's start are zeros)."""
     lib = library.core_library()
     c, taps = weight.shape
     _rows_f32(u, c, "short_conv")
-    _dev(weight, bias, state, token_seg, seg_q_start, token_slot)
+    _dev(weight, bias, state, token_seg, seg_q_start, token_slot, in_bias)
+    _need(in_bias is None or in_bias.shape == (c,), "short_conv: in_bias")
     _i32(token_seg, "token_seg"), _i32(seg_q_start, "seg_q_start"), _i32(token_slot, "token_slot")
     n = u.shape[0]
     _need(state.dtype == torch.float32 and state.dim() == 3 and state.shape[1:] == (taps - 1, c), "short_conv: state rows")
@@ -1022,24 +1025,26 @@ def short_conv(u: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None,
     _need(token_seg.numel() == n and token_slot.numel() == n, "short_conv: one segment and slot a token")
     y = torch.empty((n, c), dtype=out_dtype, device=u.device)
     _check(lib, lib.hal_short_conv(
-        _ptr(u), u.stride(0), _ptr(weight), _ptr(bias), dtype_code(weight.dtype), taps, _ptr(state), _ptr(token_seg),
+        _ptr(u), u.stride(0), _ptr(weight), _ptr(bias), dtype_code(weight.dtype), _ptr(in_bias),
+        F32 if in_bias is None else dtype_code(in_bias.dtype), taps, _ptr(state), _ptr(token_seg),
         _ptr(seg_q_start), _ptr(token_slot), _ptr(y), c, dtype_code(out_dtype), 1 if silu else 0, n, c, _stream()))
     return y
 
 
 def short_conv_through(u: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, state: torch.Tensor,
-                       ctx, out_dtype: torch.dtype, silu: bool = False) -> torch.Tensor:
+                       ctx, out_dtype: torch.dtype, silu: bool = False, in_bias: torch.Tensor | None = None) -> torch.Tensor:
     """``short_conv`` and ``short_conv_carry`` for the step ``ctx``: the convolution's result,
     and the state left as the next step finds it.  A step in which every request brings
     one token takes one kernel for both."""
     c, taps = weight.shape
     n = u.shape[0]
     if taps == 1:
-        return short_conv(u, weight, bias, state, ctx.token_seg, ctx.seg_q_start, ctx.token_slot, out_dtype, silu)
+        return short_conv(u, weight, bias, state, ctx.token_seg, ctx.seg_q_start, ctx.token_slot, out_dtype, silu, in_bias)
     if n == ctx.n_segs:
         lib = library.core_library()
         _rows_f32(u, c, "short_conv")
-        _dev(weight, bias, state)
+        _dev(weight, bias, state, in_bias)
+        _need(in_bias is None or in_bias.shape == (c,), "short_conv: in_bias")
         slot = ctx.token_slot
         _dev(slot)
         _i32(slot, "token_slot")
@@ -1048,32 +1053,36 @@ def short_conv_through(u: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor
         _need(slot.numel() == n, "short_conv: one slot a token")
         y = torch.empty((n, c), dtype=out_dtype, device=u.device)
         _check(lib, lib.hal_short_conv_step(
-            _ptr(u), u.stride(0), _ptr(weight), _ptr(bias), dtype_code(weight.dtype), taps, _ptr(state), _ptr(slot),
+            _ptr(u), u.stride(0), _ptr(weight), _ptr(bias), dtype_code(weight.dtype), _ptr(in_bias),
+            F32 if in_bias is None else dtype_code(in_bias.dtype), taps, _ptr(state), _ptr(slot),
             _ptr(y), c, dtype_code(out_dtype), 1 if silu else 0, n, c, _stream()))
         return y
-    y = short_conv(u, weight, bias, state, ctx.token_seg, ctx.seg_q_start, ctx.token_slot, out_dtype, silu)
-    short_conv_carry(u, state, ctx.seg_q_start, ctx.seg_q_len, ctx.token_slot)
+    y = short_conv(u, weight, bias, state, ctx.token_seg, ctx.seg_q_start, ctx.token_slot, out_dtype, silu, in_bias)
+    short_conv_carry(u, state, ctx.seg_q_start, ctx.seg_q_len, ctx.token_slot, in_bias)
     return y
 
 
 def short_conv_carry(u: torch.Tensor, state: torch.Tensor, seg_q_start: torch.Tensor, seg_q_len: torch.Tensor,
-                     token_slot: torch.Tensor) -> None:
+                     token_slot: torch.Tensor, in_bias: torch.Tensor | None = None) -> None:
     """After ``short_conv``: every request's state becomes the last ``taps - 1`` of (its
     state, then its inputs of this step)."""
     lib = library.core_library()
     c = state.shape[2]
     _rows_f32(u, c, "short_conv_carry")
-    _dev(state, seg_q_start, seg_q_len, token_slot)
+    _dev(state, seg_q_start, seg_q_len, token_slot, in_bias)
     _need(state.dtype == torch.float32 and state.dim() == 3, "short_conv_carry: state rows")
     _need(seg_q_start.numel() == seg_q_len.numel(), "short_conv_carry: segment arrays")
-    _check(lib, lib.hal_short_conv_carry(_ptr(u), u.stride(0), _ptr(state), state.shape[1] + 1, _ptr(seg_q_start),
+    _check(lib, lib.hal_short_conv_carry(_ptr(u), u.stride(0), _ptr(in_bias),
+                                         F32 if in_bias is None else dtype_code(in_bias.dtype),
+                                         _ptr(state), state.shape[1] + 1, _ptr(seg_q_start),
                                          _ptr(seg_q_len), _ptr(token_slot), seg_q_start.numel(), c, _stream()))
 
 
 def ssd_scan(xbc: torch.Tensor, dt_raw: torch.Tensor, dt_bias: torch.Tensor, a_log: torch.Tensor,
              d_skip: torch.Tensor, state: torch.Tensor, seg_q_start: torch.Tensor, seg_q_len: torch.Tensor,
              token_slot: torch.Tensor, groups: int, chunks: torch.Tensor | None = None,
-             seg_chunks: torch.Tensor | None = None, fixed_decay: torch.Tensor | None = None) -> torch.Tensor:
+             seg_chunks: torch.Tensor | None = None, fixed_decay: torch.Tensor | None = None,
+             in_silu: bool = False) -> torch.Tensor:
     """The state-space recurrence over every request's tokens of the step.  ``xbc``
     ``[T, heads * P + 2 * groups * N]``: x, then B and C; ``dt_raw`` float32 ``[T, heads]``
     (a row-strided view is allowed); ``state`` float32 ``[slots, heads, N, P]``, read and
@@ -1083,9 +1092,11 @@ def ssd_scan(xbc: torch.Tensor, dt_raw: torch.Tensor, dt_bias: torch.Tensor, a_l
     prompts need to fill the chip); without them a wave walks a whole segment.
     ``fixed_decay`` float32 ``[heads]``: one constant decay a head, every step size 1 and nothing
     added for the token itself (``dt_raw``, ``dt_bias``, ``a_log`` and ``d_skip`` are None):
-    ``S <- decay S + B x^T``, ``y = S^T C``."""
+    ``S <- decay S + B x^T``, ``y = S^T C``.  ``in_silu``: x, B and C are SiLU of what ``xbc``
+    holds.  ``xbc`` may be a row-strided view."""
     lib = library.core_library()
-    _dev(xbc, dt_bias, a_log, d_skip, state, seg_q_start, seg_q_len, token_slot, fixed_decay)
+    _dev(dt_bias, a_log, d_skip, state, seg_q_start, seg_q_len, token_slot, fixed_decay)
+    _need(xbc.is_cuda and xbc.dim() == 2 and xbc.stride(1) == 1, "ssd_scan: rows on the GPU")
     _, heads, n_state, p = state.shape
     n = xbc.shape[0]
     _need(state.dtype == torch.float32 and xbc.dim() == 2 and xbc.shape[1] == heads * p + 2 * groups * n_state,
@@ -1110,10 +1121,10 @@ def ssd_scan(xbc: torch.Tensor, dt_raw: torch.Tensor, dt_bias: torch.Tensor, a_l
         sums = torch.empty((n_chunks, heads, n_state, p), dtype=torch.float32, device=xbc.device)
         decays = torch.empty((n_chunks, heads), dtype=torch.float32, device=xbc.device)
     _check(lib, lib.hal_ssd_scan(
-        _ptr(xbc), xbc.shape[1], dtype_code(xbc.dtype), _ptr(dt_raw), 0 if dt_raw is None else dt_raw.stride(0),
+        _ptr(xbc), xbc.stride(0), dtype_code(xbc.dtype), _ptr(dt_raw), 0 if dt_raw is None else dt_raw.stride(0),
         _ptr(dt_bias), _ptr(a_log), _ptr(d_skip), F32 if a_log is None else dtype_code(a_log.dtype), _ptr(state), _ptr(seg_q_start), _ptr(seg_q_len), _ptr(token_slot),
         _ptr(y), seg_q_start.numel(), heads, p, n_state, groups, _ptr(chunks), _ptr(seg_chunks), n_chunks,
-        _ptr(sums), _ptr(decays), _ptr(fixed_decay), _stream()))
+        _ptr(sums), _ptr(decays), _ptr(fixed_decay), 1 if in_silu else 0, _stream()))
     return y
 
 

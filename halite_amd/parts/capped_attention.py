@@ -168,13 +168,14 @@ class CappedAttention(Mixer):
         D = self.head_dim
         a = ops.linear(x, self.w_in, out_dtype=torch.float32, tiled=self.t_in)
         qkv, gate = a[:, : self.n_conv], a[:, self.n_conv :]
-        if self.w_bias is not None:
-            ops.bias_rows_(qkv, self.w_bias)
+        # (the biases go into the convolution's reads; without a convolution a pass of their own adds them)
         if p.conv_taps is not None and p.conv_taps > 1:
-            qkv = ops.short_conv_through(qkv, self.w_conv, None, run.state["conv"], ctx, torch.float32)
+            qkv = ops.short_conv_through(qkv, self.w_conv, None, run.state["conv"], ctx, torch.float32, in_bias=self.w_bias)
         elif p.conv_taps == 1:
             qkv = ops.short_conv(qkv, self.w_conv, None, a.new_zeros((1, 0, self.n_conv)), ctx.token_seg, ctx.seg_q_start,
-                                 ctx.token_slot, torch.float32)
+                                 ctx.token_slot, torch.float32, in_bias=self.w_bias)
+        elif self.w_bias is not None:
+            ops.bias_rows_(qkv, self.w_bias)
         q, k, v = qkv[:, : self.n_q], qkv[:, self.n_q : self.n_q + self.n_k], qkv[:, self.n_q + self.n_k :]
         other = None
         if p.value_mix is not None:

@@ -98,8 +98,8 @@ class DecayAttention(Mixer):
         p = self.p
         n_act = self.inner + 2 * self.n_qk
         a = ops.linear(x, self.w_in, out_dtype=torch.float32, tiled=self.t_in)
-        vkq = ops.silu_rows(a[:, :n_act], x.dtype)
-        y = ops.ssd_scan(vkq, None, None, None, None, run.state["state"], ctx.seg_q_start, ctx.seg_q_len,
-                         ctx.token_slot, p.n_heads, fixed_decay=self.decay, **scan_arrays(ctx))
+        # (SiLU of values, keys and queries where the scan reads them: float32 in either mode)
+        y = ops.ssd_scan(a[:, :n_act], None, None, None, None, run.state["state"], ctx.seg_q_start, ctx.seg_q_len,
+                         ctx.token_slot, p.n_heads, fixed_decay=self.decay, in_silu=True, **scan_arrays(ctx))
         gated = ops.head_norm_gate(y, a[:, n_act:], self.w_norm, p.eps, 1, x.dtype)
         return ops.linear(gated, self.w_out, out_dtype=torch.float32, tiled=self.t_out)

@@ -139,9 +139,11 @@ def test_constant_decays_in_steps(gpu, stored, shape):
     assert at == T and bool(torch.isnan(state[1]).all()) and bool(torch.isnan(state[3]).all())
 
 
-def test_constant_decays_over_chunks(gpu):
+@pytest.mark.parametrize("in_silu", [False, True])
+def test_constant_decays_over_chunks(gpu, in_silu):
     """A long portion cut into chunks that are walked side by side and joined by a carry,
-    beside a short one, on states that are not zero; then single tokens on top."""
+    beside a short one, on states that are not zero; then single tokens on top.  With
+    ``in_silu`` the rows are a view into wider float32 rows and go through SiLU as they are read."""
     H, N, Pv, chunk = 3, 24, 40, 64
     T = {1: 301, 3: 70}
     decay = torch.tensor([0.97, 1.0, 0.999], dtype=F)
@@ -150,7 +152,7 @@ def test_constant_decays_over_chunks(gpu):
     state = start.clone().to(gpu)
     want = {}
     for s, a in rows.items():
-        b = a.to(F)
+        b = P.silu(a.to(F)) if in_silu else a.to(F)
         v, k, q = b[:, : H * Pv].view(-1, H, Pv), b[:, H * Pv : H * Pv + H * N].view(-1, H, N), b[:, H * Pv + H * N :].view(-1, H, N)
         want[s] = P.decayed_state_walk(q, k, v, decay, start[s].to(F))[0].reshape(T[s], H * Pv)
     at = {1: 0, 3: 0}
@@ -158,6 +160,8 @@ def test_constant_decays_over_chunks(gpu):
         slots = list(step)
         cuts = [step[s] for s in slots]
         a = torch.cat([rows[s][at[s] : at[s] + step[s]] for s in slots]).to(gpu)
+        if in_silu:
+            a = torch.cat([a, torch.full((a.shape[0], 7), float("nan"), device=gpu)], 1)[:, : H * Pv + 2 * H * N]
         _, starts, lens, slot = step_arrays(gpu, cuts, slots)
         chunks = seg_chunks = None
         if max(cuts) >= 2 * chunk:
@@ -167,7 +171,7 @@ def test_constant_decays_over_chunks(gpu):
             chunks = torch.tensor(rows_, dtype=torch.int32, device=gpu)
             seg_chunks = torch.tensor([[f, n] for f, n in zip(first, per)], dtype=torch.int32, device=gpu)
         y = ops.ssd_scan(a, None, None, None, None, state, starts, lens, slot, H, fixed_decay=decay.float().to(gpu),
-                         chunks=chunks, seg_chunks=seg_chunks).cpu()
+                         chunks=chunks, seg_chunks=seg_chunks, in_silu=in_silu).cpu()
         i = 0
         for s in slots:
             ref = want[s][at[s] : at[s] + step[s]]
