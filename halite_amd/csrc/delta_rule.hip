@@ -472,12 +472,43 @@ __global__ void head_norm_gate_kernel(const float* __restrict__ y, const float* 
   }
 }
 
+// The same for heads of many channels: a workgroup a (token, head).
+template <typename T>
+__global__ void __launch_bounds__(256)
+head_norm_gate_wide_kernel(const float* __restrict__ y, const float* __restrict__ z, int ldz,
+                           const void* __restrict__ w, int w_dtype, float eps, T* __restrict__ out, int H, int D) {
+  __shared__ float scratch[16];
+  const size_t t = blockIdx.x;
+  const int h = blockIdx.y;
+  const float* yr = y + (t * H + h) * D;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < D; i += blockDim.x) ss += yr[i] * yr[i];
+  const float rstd = 1.0f / sqrtf(block_sum(ss, scratch) / (float)D + eps);
+  for (int i = threadIdx.x; i < D; i += blockDim.x) {
+    const size_t c = (size_t)h * D + i;
+    const float g = z ? delta_sigmoid(z[t * ldz + c]) : 1.0f;
+    const float wt = w ? load_as_f32(w, w_dtype, c) : 1.0f;
+    out[t * H * D + c] = from_f32<T>(yr[i] * rstd * wt * g);
+  }
+}
+
 extern "C" int hal_head_norm_gate(const float* y, const float* z, int ldz, const void* w, int w_dtype, float eps,
                                   void* out, int dtype, int n_tokens, int H, int D, hipStream_t stream) {
   HAL_REQUIRE(n_tokens >= 0 && H > 0 && D > 0 && (z == nullptr || ldz >= H * D),
               "hal_head_norm_gate: bad sizes T=%d heads=%d dim=%d", n_tokens, H, D);
   HAL_REQUIRE(dtype == HAL_F32 || dtype == HAL_BF16, "hal_head_norm_gate: dtype %d", dtype);
   if (n_tokens == 0) return 0;
+  if (D >= 512 && H <= 65535) {
+    const dim3 wide(n_tokens, H);
+    if (dtype == HAL_F32)
+      hipLaunchKernelGGL(head_norm_gate_wide_kernel<float>, wide, dim3(256), 0, stream, y, z, ldz, w, w_dtype, eps,
+                         (float*)out, H, D);
+    else
+      hipLaunchKernelGGL(head_norm_gate_wide_kernel<bf16_t>, wide, dim3(256), 0, stream, y, z, ldz, w, w_dtype, eps,
+                         (bf16_t*)out, H, D);
+    HAL_LAUNCH_CHECK();
+    return 0;
+  }
   const long long units = (long long)n_tokens * H;
   const dim3 grid((unsigned)((units + 3) / 4));
   if (dtype == HAL_F32)

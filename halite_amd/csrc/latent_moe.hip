@@ -311,7 +311,8 @@ __global__ void moe_combine_kernel(float* __restrict__ h, const float* __restric
                                    const float* __restrict__ extra_gate, int ld_gate, int top, int d) {
   const int t = blockIdx.x;
   const float eg = extra_gate ? 1.0f / (1.0f + expf(-extra_gate[(size_t)t * ld_gate])) : 1.0f;
-  for (int i = threadIdx.x; i < d; i += blockDim.x) {
+  // (a step of few tokens spreads a row over several workgroups: blockIdx.y takes every gridDim.y-th run of columns)
+  for (int i = blockIdx.y * blockDim.x + threadIdx.x; i < d; i += blockDim.x * gridDim.y) {
     float s = extra ? eg * extra[(size_t)t * d + i] : 0.f;
     for (int j = 0; j < top; ++j) s += wgt[(size_t)t * top + j] * y[((size_t)t * top + j) * d + i];
     h[(size_t)t * d + i] += s;
@@ -325,7 +326,9 @@ extern "C" int hal_moe_combine(float* h, const float* y, const float* wgt, const
   if (n_tokens == 0) return 0;
   int threads = (d + 63) / 64 * 64;
   if (threads > 256) threads = 256;
-  hipLaunchKernelGGL(moe_combine_kernel, dim3(n_tokens), dim3(threads), 0, stream, h, y, wgt, extra, extra_gate, ld_gate, top, d);
+  int parts = 1;  // workgroups a row, so that a decode step has a few hundred of them
+  while (parts < 16 && n_tokens * parts < 256 && d / (threads * parts * 2) >= 1) parts *= 2;
+  hipLaunchKernelGGL(moe_combine_kernel, dim3(n_tokens, parts), dim3(threads), 0, stream, h, y, wgt, extra, extra_gate, ld_gate, top, d);
   HAL_LAUNCH_CHECK();
   return 0;
 }

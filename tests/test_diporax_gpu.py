@@ -248,6 +248,31 @@ def test_routing_weights_and_gates(gpu):
     assert float((hg.cpu() - want).abs().max()) < 1e-5
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("shape", [(1, 1100), (3, 512), (1, 96), (2, 4096)])
+def test_rows_normed_weighted_and_gated(gpu, dtype, shape):
+    """The heads of a row (one head: the whole row) divided by their root mean square, times a
+    weight and the sigmoid of a gate; narrow heads a wave each, wide ones a workgroup each."""
+    H, D = shape
+    t = 9
+    y, a = rand(t, H * D, seed=1, scale=3.0), rand(t, 5 + H * D, seed=2)
+    w = (1 + 0.2 * rand(H * D, seed=3)).to(DT[dtype])
+    got = ops.head_norm_gate(y.to(gpu), a.to(gpu)[:, 5:], w.to(gpu), 1e-5, H, DT[dtype]).float().cpu()
+    want = P.rms_unit(y.to(F).view(t, H, D), 1e-5).reshape(t, H * D) * w.to(F) * torch.sigmoid(a[:, 5:].to(F))
+    assert float((got - want).abs().max()) < (1e-5 if dtype == "float32" else 2e-2) * float(want.abs().max())
+
+
+@pytest.mark.parametrize("sizes", [(3, 4096, 4), (70, 40, 2), (300, 1024, 1), (1, 520, 3)])
+def test_weighted_sum_of_the_chosen_experts(gpu, sizes):
+    """Few tokens spread a row over several workgroups, many take one each: the same sums."""
+    t, d, top = sizes
+    h, y, wgt, extra, g = rand(t, d, seed=1), rand(t * top, d, seed=2), rand(t, top, seed=3).abs(), rand(t, d, seed=4), rand(t, 1, seed=5)
+    hg = h.to(gpu)
+    ops.moe_combine(hg, y.to(gpu), wgt.to(gpu), extra.to(gpu), extra_gate=g.to(gpu))
+    want = h.to(F) + (wgt.to(F)[:, :, None] * y.to(F).view(t, top, d)).sum(1) + torch.sigmoid(g.to(F)) * extra.to(F)
+    assert float((hg.cpu() - want).abs().max()) < 1e-5
+
+
 def test_stretched_rotation_tables(gpu):
     """The rotary part's table against the plain frequencies: the ramp between fast and slow
     pairs, and cosine and sine times the stretch's magnitude."""
