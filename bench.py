@@ -99,7 +99,7 @@ class Families:
     GEMM = ("linear", "linear_add", "gemm_bf16_skinny", "gemm_bf16_skinny_norm", "qkv_rope_append", "gemm_f32")
     GROUPED = ("grouped_gemm",)
     ELEMENTWISE = ("rmsnorm", "silu_mul", "rope_append", "embedding", "residual_add", "rmsnorm_exact", "latent_prep",
-                   "head_cols", "scale_", "moe_route", "moe_sort", "moe_combine", "clamped_gate_mul", "cast_rows",
+                   "head_cols", "scale_", "moe_route", "moe_sort", "moe_route_sort", "moe_combine", "clamped_gate_mul", "cast_rows",
                    "post_norm_add", "relu_squared", "scaled_sum_", "qk_norm_pack", "gated_part_norm", "head_norm_gate",
                    "streams_step", "head_norm_pack", "head_gate_cols", "bias_rows_", "silu_rows", "token_gate")
     RECURRENT = ("short_conv", "short_conv_carry", "ssd_scan", "delta_rule")

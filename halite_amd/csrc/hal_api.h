@@ -185,10 +185,14 @@ int hal_moe_route(const float* z, int ldz, int E, int top, int softmax, int norm
 int hal_moe_sort(const int* idx, int n, int E, int tile, int* offsets, int* tile_offsets,
                  int* sorted, hipStream_t stream);
 // h[t] += sum_j wgt[t, j] * y[t * top + j] (+ extra[t] if given, times sigmoid(extra_gate[t *
-// ld_gate]) if that is given)  (h, extra [T, d] and y [T * top, d] float32)
+// ld_gate]) if that is given)  (h, extra [T, d] and y [T * top, d] float32); overwrite: h[t] = the sum
 int hal_moe_combine(float* h, const float* y, const float* wgt, const float* extra,
-                    const float* extra_gate, int ld_gate, int top, int d, int n_tokens,
+                    const float* extra_gate, int ld_gate, int top, int d, int n_tokens, int overwrite,
                     hipStream_t stream);
+// hal_moe_route and hal_moe_sort in one workgroup (for steps of few tokens)
+int hal_moe_route_sort(const float* z, int ldz, int E, int top, int softmax, int normalize, float norm_eps,
+                       int* idx, float* wgt, int n_tokens, int tile, int* offsets, int* tile_offsets,
+                       int* sorted, hipStream_t stream);
 
 // out [T, F] = g * sigmoid(alpha * g) * (u + up_shift), g = min(gu[t, f], limit), u = clamp(gu[t, F + f],
 // -limit, limit), for rows gu [T, 2F] that hold a gate projection and an up projection.

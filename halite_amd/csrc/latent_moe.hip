@@ -184,10 +184,9 @@ extern "C" int hal_scale_f32(float* x, long long n, float s, hipStream_t stream)
 // One wave a token: lane l holds the scores of the experts l, l + 64, ...; each of the `top`
 // rounds finds the largest score that is left (the lower index on a tie) across the wave.
 #define MOE_ROUTE_PER_LANE (MOE_MAX_EXPERTS / HAL_WAVE)
-__global__ void __launch_bounds__(HAL_WAVE) moe_route_kernel(const float* __restrict__ z, int ldz, int E, int top, int softmax,
-                                                             int normalize, float norm_eps, int* __restrict__ idx,
-                                                             float* __restrict__ wgt, int n_tokens) {
-  const int t = blockIdx.x, lane = threadIdx.x;
+__device__ __forceinline__ void moe_route_token(const float* __restrict__ z, int ldz, int E, int top, int softmax,
+                                                int normalize, float norm_eps, int* __restrict__ idx,
+                                                float* __restrict__ wgt, int t, int lane) {
   const float* zr = z + (size_t)t * ldz;
   float s[MOE_ROUTE_PER_LANE];
   float zmax = -INFINITY;
@@ -243,6 +242,12 @@ __global__ void __launch_bounds__(HAL_WAVE) moe_route_kernel(const float* __rest
   }
 }
 
+__global__ void __launch_bounds__(HAL_WAVE) moe_route_kernel(const float* __restrict__ z, int ldz, int E, int top, int softmax,
+                                                             int normalize, float norm_eps, int* __restrict__ idx,
+                                                             float* __restrict__ wgt, int n_tokens) {
+  moe_route_token(z, ldz, E, top, softmax, normalize, norm_eps, idx, wgt, blockIdx.x, threadIdx.x);
+}
+
 extern "C" int hal_moe_route(const float* z, int ldz, int E, int top, int softmax, int normalize,
                              float norm_eps, int* idx, float* wgt, int n_tokens,
                              hipStream_t stream) {
@@ -262,12 +267,10 @@ extern "C" int hal_moe_route(const float* z, int ldz, int E, int top, int softma
 // choice), expert by expert.  The order inside an expert is not fixed; nothing that is
 // computed from it depends on it.
 // ---------------------------------------------------------------------------------
-__global__ void __launch_bounds__(1024) moe_sort_kernel(const int* __restrict__ idx, int n, int E, int tile,
-                                                        int* __restrict__ offsets,
-                                                        int* __restrict__ tile_offsets,
-                                                        int* __restrict__ sorted) {
-  __shared__ int count[MOE_MAX_EXPERTS];
-  __shared__ int cursor[MOE_MAX_EXPERTS];
+// (idx without __restrict__: the kernel that routes and sorts in one has just written it)
+__device__ __forceinline__ void moe_sort_pairs(const int* idx, int n, int E, int tile,
+                                               int* __restrict__ offsets, int* __restrict__ tile_offsets,
+                                               int* __restrict__ sorted, int* count, int* cursor) {
   for (int e = threadIdx.x; e < E; e += blockDim.x) count[e] = 0;
   __syncthreads();
   for (int i = threadIdx.x; i < n; i += blockDim.x) {
@@ -294,6 +297,43 @@ __global__ void __launch_bounds__(1024) moe_sort_kernel(const int* __restrict__ 
   }
 }
 
+__global__ void __launch_bounds__(1024) moe_sort_kernel(const int* __restrict__ idx, int n, int E, int tile,
+                                                        int* __restrict__ offsets,
+                                                        int* __restrict__ tile_offsets,
+                                                        int* __restrict__ sorted) {
+  __shared__ int count[MOE_MAX_EXPERTS];
+  __shared__ int cursor[MOE_MAX_EXPERTS];
+  moe_sort_pairs(idx, n, E, tile, offsets, tile_offsets, sorted, count, cursor);
+}
+
+// Both in one workgroup, for steps of few tokens: its sixteen waves take the tokens in turn,
+// then all of it sorts the pairs.
+__global__ void __launch_bounds__(1024) moe_route_sort_kernel(const float* __restrict__ z, int ldz, int E, int top,
+                                                              int softmax, int normalize, float norm_eps,
+                                                              int* __restrict__ idx, float* __restrict__ wgt,
+                                                              int n_tokens, int tile, int* __restrict__ offsets,
+                                                              int* __restrict__ tile_offsets, int* __restrict__ sorted) {
+  __shared__ int count[MOE_MAX_EXPERTS];
+  __shared__ int cursor[MOE_MAX_EXPERTS];
+  const int wave = threadIdx.x / HAL_WAVE, lane = threadIdx.x % HAL_WAVE;
+  for (int t = wave; t < n_tokens; t += 1024 / HAL_WAVE)
+    moe_route_token(z, ldz, E, top, softmax, normalize, norm_eps, idx, wgt, t, lane);
+  __threadfence_block();
+  __syncthreads();
+  moe_sort_pairs(idx, n_tokens * top, E, tile, offsets, tile_offsets, sorted, count, cursor);
+}
+
+extern "C" int hal_moe_route_sort(const float* z, int ldz, int E, int top, int softmax, int normalize, float norm_eps,
+                                  int* idx, float* wgt, int n_tokens, int tile, int* offsets, int* tile_offsets,
+                                  int* sorted, hipStream_t stream) {
+  HAL_REQUIRE(n_tokens >= 0 && E > 0 && E <= MOE_MAX_EXPERTS && top > 0 && top <= E && ldz >= E && tile > 0,
+              "hal_moe_route_sort: bad sizes T=%d E=%d top=%d", n_tokens, E, top);
+  hipLaunchKernelGGL(moe_route_sort_kernel, dim3(1), dim3(1024), 0, stream, z, ldz, E, top, softmax, normalize, norm_eps,
+                     idx, wgt, n_tokens, tile, offsets, tile_offsets, sorted);
+  HAL_LAUNCH_CHECK();
+  return 0;
+}
+
 extern "C" int hal_moe_sort(const int* idx, int n, int E, int tile, int* offsets, int* tile_offsets,
                             int* sorted, hipStream_t stream) {
   HAL_REQUIRE(n >= 0 && E > 0 && E <= MOE_MAX_EXPERTS && tile > 0, "hal_moe_sort: bad sizes n=%d E=%d", n, E);
@@ -308,27 +348,27 @@ extern "C" int hal_moe_sort(const int* idx, int n, int E, int tile, int* offsets
 // ---------------------------------------------------------------------------------
 __global__ void moe_combine_kernel(float* __restrict__ h, const float* __restrict__ y,
                                    const float* __restrict__ wgt, const float* __restrict__ extra,
-                                   const float* __restrict__ extra_gate, int ld_gate, int top, int d) {
+                                   const float* __restrict__ extra_gate, int ld_gate, int top, int d, bool overwrite) {
   const int t = blockIdx.x;
   const float eg = extra_gate ? 1.0f / (1.0f + expf(-extra_gate[(size_t)t * ld_gate])) : 1.0f;
   // (a step of few tokens spreads a row over several workgroups: blockIdx.y takes every gridDim.y-th run of columns)
   for (int i = blockIdx.y * blockDim.x + threadIdx.x; i < d; i += blockDim.x * gridDim.y) {
     float s = extra ? eg * extra[(size_t)t * d + i] : 0.f;
     for (int j = 0; j < top; ++j) s += wgt[(size_t)t * top + j] * y[((size_t)t * top + j) * d + i];
-    h[(size_t)t * d + i] += s;
+    h[(size_t)t * d + i] = overwrite ? s : h[(size_t)t * d + i] + s;
   }
 }
 
 extern "C" int hal_moe_combine(float* h, const float* y, const float* wgt, const float* extra,
                                const float* extra_gate, int ld_gate, int top, int d, int n_tokens,
-                               hipStream_t stream) {
+                               int overwrite, hipStream_t stream) {
   HAL_REQUIRE(n_tokens >= 0 && top > 0 && d > 0, "hal_moe_combine: bad sizes");
   if (n_tokens == 0) return 0;
   int threads = (d + 63) / 64 * 64;
   if (threads > 256) threads = 256;
   int parts = 1;  // workgroups a row, so that a decode step has a few hundred of them
   while (parts < 16 && n_tokens * parts < 256 && d / (threads * parts * 2) >= 1) parts *= 2;
-  hipLaunchKernelGGL(moe_combine_kernel, dim3(n_tokens, parts), dim3(threads), 0, stream, h, y, wgt, extra, extra_gate, ld_gate, top, d);
+  hipLaunchKernelGGL(moe_combine_kernel, dim3(n_tokens, parts), dim3(threads), 0, stream, h, y, wgt, extra, extra_gate, ld_gate, top, d, overwrite != 0);
   HAL_LAUNCH_CHECK();
   return 0;
 }

@@ -853,6 +853,27 @@ def moe_route(z: torch.Tensor, top: int, softmax: bool = False, normalize: bool 
     return idx, wgt
 
 
+ROUTE_SORT_MAX_TOKENS = 128  # up to so many tokens one workgroup routes and sorts
+
+
+def moe_route_sort(z: torch.Tensor, top: int, n_experts: int, softmax: bool = False, normalize: bool = True,
+                   norm_eps: float = 0.0):
+    """``moe_route`` and ``moe_sort`` in one launch: ``(idx, wgt, offsets, tile_offsets, sorted)``."""
+    lib = library.core_library()
+    _need(z.is_cuda and z.dtype == torch.float32 and z.dim() == 2 and z.stride(1) == 1 and z.shape[1] == n_experts,
+          "moe_route_sort: float32 logits [T, E] (a row-strided view is allowed)")
+    t = z.shape[0]
+    idx = torch.empty((t, top), dtype=torch.int32, device=z.device)
+    wgt = torch.empty((t, top), dtype=torch.float32, device=z.device)
+    offsets = torch.empty(n_experts + 1, dtype=torch.int32, device=z.device)
+    tile_offsets = torch.empty(n_experts + 1, dtype=torch.int32, device=z.device)
+    order = torch.empty(max(t * top, 1), dtype=torch.int32, device=z.device)
+    _check(lib, lib.hal_moe_route_sort(_ptr(z), z.stride(0), n_experts, top, 1 if softmax else 0, 1 if normalize else 0,
+                                       ctypes.c_float(norm_eps), _ptr(idx), _ptr(wgt), t, GROUP_TILE_ROWS, _ptr(offsets),
+                                       _ptr(tile_offsets), _ptr(order), _stream()))
+    return idx, wgt, offsets, tile_offsets, order
+
+
 def moe_sort(idx: torch.Tensor, n_experts: int):
     """The (token, choice) pairs of ``idx`` ``[T, top]`` sorted by expert on the device:
     ``offsets`` and ``tile_offsets`` ``[E + 1]`` and ``sorted`` ``[T * top]`` (pair numbers
@@ -869,10 +890,10 @@ def moe_sort(idx: torch.Tensor, n_experts: int):
 
 
 def moe_combine(h: torch.Tensor, y: torch.Tensor, wgt: torch.Tensor, extra: torch.Tensor | None = None,
-                extra_gate: torch.Tensor | None = None) -> None:
+                extra_gate: torch.Tensor | None = None, overwrite: bool = False) -> None:
     """``h[t] += sum_j wgt[t, j] * y[t * top + j] (+ extra[t])`` (all float32); with
     ``extra_gate`` (float32 ``[T, 1]``, a row-strided view is allowed) ``extra[t]`` is
-    multiplied by ``sigmoid(extra_gate[t])``."""
+    multiplied by ``sigmoid(extra_gate[t])``.  ``overwrite``: ``h[t]`` becomes the sum (what it held is not read)."""
     lib = library.core_library()
     _dev(h, y, wgt, extra)
     t, top = wgt.shape
@@ -883,7 +904,8 @@ def moe_combine(h: torch.Tensor, y: torch.Tensor, wgt: torch.Tensor, extra: torc
         _need(extra is not None and extra_gate.is_cuda and extra_gate.dtype == torch.float32
               and extra_gate.shape == (t, 1), "moe_combine: a float32 gate [T, 1] for the extra rows")
     _check(lib, lib.hal_moe_combine(_ptr(h), _ptr(y), _ptr(wgt), _ptr(extra), _ptr(extra_gate),
-                                    0 if extra_gate is None else extra_gate.stride(0), top, h.shape[1], t, _stream()))
+                                    0 if extra_gate is None else extra_gate.stride(0), top, h.shape[1], t,
+                                    1 if overwrite else 0, _stream()))
 
 
 def clamped_gate_mul(gate_up: torch.Tensor, limit: float, alpha: float, up_shift: float = 1.0) -> torch.Tensor:

@@ -140,12 +140,16 @@ class MixtureOfExperts(FeedForward):
     def forward(self, x, ctx, add_to=None):
         p = self.p
         n, d = x.shape
-        h = add_to if add_to is not None else torch.zeros((n, d), dtype=torch.float32, device=x.device)
+        h = add_to if add_to is not None else torch.empty((n, d), dtype=torch.float32, device=x.device)
         z = ops.linear(x, self.w_router, out_dtype=torch.float32)
         shared_gate = z[:, p.n_experts:] if p.shared_gate else None
         z = z[:, : p.n_experts]
-        idx, wgt = ops.moe_route(z, p.top_k, softmax=p.score == "softmax", normalize=p.normalize, norm_eps=p.norm_eps)
-        offsets, tiles, order = ops.moe_sort(idx, p.n_experts)
+        routing = dict(softmax=p.score == "softmax", normalize=p.normalize, norm_eps=p.norm_eps)
+        if n <= ops.ROUTE_SORT_MAX_TOKENS:  # few tokens: one workgroup routes and sorts
+            idx, wgt, offsets, tiles, order = ops.moe_route_sort(z, p.top_k, p.n_experts, **routing)
+        else:
+            idx, wgt = ops.moe_route(z, p.top_k, **routing)
+            offsets, tiles, order = ops.moe_sort(idx, p.n_experts)
         pairs = n * p.top_k
         # rows in the sorted order: row i belongs to pair order[i] = token * top_k + choice
         act = torch.empty((pairs, p.expert.intermediate_size), dtype=x.dtype, device=x.device)
@@ -169,7 +173,8 @@ class MixtureOfExperts(FeedForward):
                                             p.shared.up_shift)
             # the shared expert's result rides along with the weighted sum
             extra = ops.linear(acts, self.ws_down, out_dtype=torch.float32, tiled=self.t_shared_down)
-        ops.moe_combine(h, y, wgt, extra if p.shared is not None else None, extra_gate=shared_gate)
+        ops.moe_combine(h, y, wgt, extra if p.shared is not None else None, extra_gate=shared_gate,
+                        overwrite=add_to is None)
         if add_to is not None:
             return None
         return h if p.float32_result else h.to(x.dtype)

@@ -238,6 +238,13 @@ def test_routing_weights_and_gates(gpu):
     chosen = torch.topk(z[:, :E].to(F), top, dim=-1)
     assert torch.equal(idx.cpu().long(), chosen.indices)
     assert float((wgt.cpu() - torch.softmax(chosen.values, -1)).abs().max()) < 1e-6
+    # the same, and the pairs sorted by expert, from one launch
+    idx2, wgt2, offsets, tiles, order = ops.moe_route_sort(z.to(gpu)[:, :E], top, E, softmax=True, normalize=True, norm_eps=0.0)
+    assert torch.equal(idx2, idx) and torch.equal(wgt2, wgt)
+    o, pairs, flat = offsets.cpu().tolist(), order.cpu().tolist(), idx.cpu().flatten().tolist()
+    assert o[0] == 0 and o[E] == t * top and sorted(pairs) == list(range(t * top))
+    assert all(flat[pairs[i]] == e for e in range(E) for i in range(o[e], o[e + 1]))
+    assert tiles.cpu().tolist() == [sum(-(-(o[j + 1] - o[j]) // ops.GROUP_TILE_ROWS) for j in range(e)) for e in range(E + 1)]
     gu = rand(t, 2 * d, seed=2, scale=3.0)
     got = ops.clamped_gate_mul(gu.to(gpu), math.inf, 1.0, 0.0).cpu()
     assert float((got - P.silu(gu[:, :d].to(F)) * gu[:, d:].to(F)).abs().max()) < 1e-5
@@ -271,6 +278,9 @@ def test_weighted_sum_of_the_chosen_experts(gpu, sizes):
     ops.moe_combine(hg, y.to(gpu), wgt.to(gpu), extra.to(gpu), extra_gate=g.to(gpu))
     want = h.to(F) + (wgt.to(F)[:, :, None] * y.to(F).view(t, top, d)).sum(1) + torch.sigmoid(g.to(F)) * extra.to(F)
     assert float((hg.cpu() - want).abs().max()) < 1e-5
+    fresh = torch.full((t, d), float("nan"), device=gpu)  # written, not added to
+    ops.moe_combine(fresh, y.to(gpu), wgt.to(gpu), extra.to(gpu), extra_gate=g.to(gpu), overwrite=True)
+    assert float((fresh.cpu() - (want - h.to(F))).abs().max()) < 1e-5
 
 
 def test_stretched_rotation_tables(gpu):
