@@ -853,7 +853,7 @@ def moe_route(z: torch.Tensor, top: int, softmax: bool = False, normalize: bool 
     return idx, wgt
 
 
-ROUTE_SORT_MAX_TOKENS = 128  # up to so many tokens one workgroup routes and sorts
+ROUTE_SORT_MAX_TOKENS = 16  # up to so many tokens (one a wave) one workgroup routes and sorts
 
 
 def moe_route_sort(z: torch.Tensor, top: int, n_experts: int, softmax: bool = False, normalize: bool = True,
