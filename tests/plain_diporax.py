@@ -208,12 +208,21 @@ def token_input(x, tokens, w, pre, table, eps):
 
 
 def forward(cfg: dict, w: dict, tokens, dtype=torch.float64, layers_out: list | None = None, round_inputs=None,
-            margins_out: list | None = None) -> torch.Tensor:
+            margins_out: list | None = None, disturb: float = 0.0, seed: int = 0) -> torch.Tensor:
     """Logits ``[T, vocab]`` of one request's tokens; ``layers_out`` collects the stream
     after every layer.  ``round_inputs``: an element type that every part's input is rounded
     to on the way (how far the logits move then says how sensitive a position is to arithmetic
-    in that type).  ``margins_out`` receives every router's margins (see ``routed_experts``)."""
-    rounded = (lambda t: t.to(round_inputs).to(dtype)) if round_inputs is not None else (lambda t: t)
+    in that type); ``disturb``: a relative error that every entry of every part's input is moved by,
+    drawn from ``seed``.  ``margins_out`` receives every router's margins (see ``routed_experts``)."""
+    gen = torch.Generator().manual_seed(seed)
+
+    def rounded(t):
+        if round_inputs is not None:
+            t = t.to(round_inputs).to(dtype)
+        if disturb:  # every entry moved by a relative error of that size (what arithmetic in 16 bits has piled up by then)
+            t = t * (1.0 + disturb * torch.randn(t.shape, generator=gen, dtype=dtype))
+        return t
+
     w = {k: (v.to(dtype) if v.is_floating_point() else v) for k, v in w.items()}
     eps = cfg["norm"]["eps"]
     tokens = torch.as_tensor(tokens, dtype=torch.long)
