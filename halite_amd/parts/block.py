@@ -103,7 +103,9 @@ class ParallelBlock(Arrangement):
 class PostNormBlock(Arrangement):
     """``h = h + norm_a(mixer(h)); h = h + norm_b(ff(h))``: the parts read the stream itself
     and the norm is on what they return.  A layer may leave the feed-forward (and its
-    norm) out.
+    norm) out, and may close with a third part of the feed-forward kind, ``side``, with a norm
+    of its own: ``h = h + norm_c(side(h))``.  A norm with a layer scale multiplies by its
+    weight times that scale (``RMSNorm.multiplier``).
 
     The parts return float32 rows; norm, weight and sum are one float32 pass
     (``ops.post_norm_add``), which also leaves the new rows rounded to the activation type
