@@ -505,7 +505,7 @@ def diporax_layer_kinds(n_layers):
 
 
 def diporax_config(s, n_layers, window):
-    rot = dict(base=500000.0, dims=64, scaling=dict(factor=4.0, original=2048, fast=32.0, slow=1.0))
+    rot = dict(base=500000.0, dims=64, scaling=dict(factor=8.0, original=4096, fast=32.0, slow=1.0))
     attention = dict(heads=s["heads"], kv_heads=s["kv_heads"], dim=s["dim"], vdim=s["dim"], scale=s["dim"] ** -0.5,
                      conv=s["conv"], rot=rot, softcap=30.0, v_mix=True, bias=True)
     latent = dict(heads=s["heads"], dim=s["dim"], rot_dim=s["rot_dim"], vdim=s["dim"], q_rank=s["q_rank"],

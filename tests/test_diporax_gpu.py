@@ -290,7 +290,7 @@ def test_stretched_rotation_tables(gpu):
     from halite_amd.parts.rope import Rope, RopeParams
 
     for r in (P.rot(1000.0, 8, factor=4.0), P.rot(77.0, 6, factor=8.0, original=16, fast=4.0, slow=0.5), P.rot(50.0, 4),
-              P.rot(250000.0, 32, factor=2.0, original=1024)):
+              P.rot(1000000.0, 48, factor=3.0, original=512, fast=16.0, slow=2.0)):
         s = r.get("scaling")
         params = RopeParams(head_dim=r["dims"], rotary_dim=r["dims"], theta=r["base"], max_positions=4096, angles="float64",
                             scaling=None if s is None else dict(kind="ramp", factor=s["factor"], original_context_len=s["original"],
